@@ -1,0 +1,146 @@
+#!/usr/bin/env python3
+"""Headline benchmark: per-token logprob over bf16 logits [G=256, L=512, V=128256] on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one compute_logp call over the whole resident [256, 512, 128256] tensor (33.6 GB),
+i.e. 131,072 tokens.  Prints ONE JSON line; `value` is tokens/s with the logits already in HBM.
+`roofline` prices the logprob kernel against the 8 TB/s HBM peak from the algorithmic bytes
+(2*V + 8 + 4 per token); `cpu_baseline` times the CPU oracle on a bounded sample of the same
+tensor on this box's host cores.  Sampling latency at batch 256 rides along in `sampling`.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+REPO = Path(__file__).resolve().parent
+for _p in (REPO, REPO / "kernel-align_amd"):
+    if str(_p) not in sys.path:
+        sys.path.insert(0, str(_p))
+
+HBM_PEAK_GBPS = 8000.0
+G, L, V = 256, 512, 128256
+BYTES_PER_TOKEN = 2 * V + 8 + 4
+
+
+def log(msg: str) -> None:
+    print(msg, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(logits, ids, sample_rows: int):
+    """Time the fp32 torch CPU oracle on `sample_rows` rows taken evenly from the tensor."""
+    import torch
+    from oracle import logprob_ref
+
+    blk = 2048
+    n_blocks = max(1, sample_rows // blk)
+    total_rows = logits.shape[0]
+    starts = [int(i * (total_rows - blk) / max(1, n_blocks - 1)) // blk * blk for i in range(n_blocks)]
+    elapsed, rows, max_err = 0.0, 0, None
+    for s in starts:
+        lc, ic = logits[s:s + blk].cpu(), ids[s:s + blk].cpu()
+        t0 = time.perf_counter()
+        logprob_ref.logprob_ref(lc, ic)
+        elapsed += time.perf_counter() - t0
+        rows += lc.shape[0]
+    return {
+        "value": rows / elapsed,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{rows} of {total_rows} tokens ({n_blocks} blocks of {blk} rows, fp32 torch CPU "
+                  f"log_softmax+gather), {elapsed:.1f} s; host cpu_count={os.cpu_count()}",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-sample-rows", type=int, default=32768,
+                    help="rows of the tensor the CPU oracle is timed on (0 = skip)")
+    ap.add_argument("--chunk-tokens", type=int, default=None, help="rows per kernel launch")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log(f"bench.py measures one GPU: --gpus {args.gpus} is not supported in this build "
+            "(token rows are independent; more GPUs would each take a slice of the rows)")
+        return 2
+
+    import torch
+    from benchmarks.workloads import spike_logits
+    from rl_engine.kernels import sampling as sampling_mod
+    from rl_engine.kernels.sampling import SamplerBackend
+
+    if not torch.cuda.is_available():
+        log("bench.py needs an MI355X: no GPU visible")
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    sampler = SamplerBackend().to(dev)
+    chunk = args.chunk_tokens or sampling_mod.DEFAULT_CHUNK_TOKENS
+
+    n_rows = G * L
+    log(f"generating bf16 logits [{G},{L},{V}] ({n_rows * V * 2 / 1e9:.1f} GB) on {torch.cuda.get_device_name(0)}")
+    logits, ids = spike_logits(n_rows, V, seed=0, device=dev)
+    logits3, ids2 = logits.view(G, L, V), ids.view(G, L)
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        sampler.compute_logp(logits3, ids2, chunk_tokens=chunk)
+    torch.cuda.synchronize()
+
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(args.steps):
+        out = sampler.compute_logp(logits3, ids2, chunk_tokens=chunk)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    launches_per_step = (n_rows + chunk - 1) // chunk
+    # The events sit on the stream the kernels were launched on (torch's current stream).
+    launch_ms = ev0.elapsed_time(ev1) / (args.steps * launches_per_step)
+    rows_per_launch = n_rows / launches_per_step
+    achieved_gbps = rows_per_launch * BYTES_PER_TOKEN / (launch_ms * 1e-3) / 1e9
+    tokens_per_s = n_rows / (ms_per_step * 1e-3)
+
+    result = {
+        "metric": "logprob tokens/s (G=256,L=512,V=128256)",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "GRPO large-group logprob: bf16 logits [256,512,128256] ~ N(0,3^2) + 1% spike "
+                               "rows, ids uniform, seed 0", "chunk_tokens": chunk,
+                   "launches_per_step": launches_per_step, "input_dtype": "bf16", "output_dtype": "f32"},
+        "hbm_gbps": n_rows * BYTES_PER_TOKEN / (ms_per_step * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "logprob_rows<Bf16,256,4,vec>", "launch_ms": launch_ms,
+                     "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
+    }
+    assert bool(torch.isfinite(out).all()), "non-finite logprob in the timed run"
+    if args.cpu_sample_rows > 0:
+        log("timing the CPU oracle on a sample of the same tensor")
+        result["cpu_baseline"] = cpu_baseline(logits, ids, args.cpu_sample_rows)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

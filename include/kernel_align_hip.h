@@ -1,0 +1,122 @@
+/*
+ * kernel_align_hip.h — C ABI of libkernel_align_hip.so (MI355X / gfx950).
+ *
+ * The library implements the data-parallel hot path of Kernel-Align as
+ * hand-written HIP kernels: the per-token logprob operator, the fused
+ * temperature / top-k / top-p sampling operator, and a fused
+ * lm_head -> logprob operator.  Every entry point takes plain device pointers
+ * and sizes, enqueues work on the caller's HIP stream and returns without
+ * synchronising.  The library never allocates or frees device memory and never
+ * keeps a pointer after the call returns; scratch space is passed in as a
+ * workspace whose size the *_workspace_bytes queries report.
+ *
+ * Return value of every int-returning entry point: KA_OK (0) or a negative
+ * KA_ERR_* code; ka_last_error() then holds a thread-local message.
+ *
+ * There is no CPU fallback in this library: without a HIP device every compute
+ * entry point returns KA_ERR_HIP.
+ */
+#ifndef KERNEL_ALIGN_HIP_H
+#define KERNEL_ALIGN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KA_OK 0
+#define KA_ERR_BAD_ARG (-1)      /* null pointer, negative size, top_k < 0, top_p outside (0,1], T <= 0 */
+#define KA_ERR_UNSUPPORTED (-2)  /* shape the kernels cannot take (e.g. vocab >= 2^31) */
+#define KA_ERR_WORKSPACE (-3)    /* workspace missing or smaller than *_workspace_bytes() */
+#define KA_ERR_HIP (-4)          /* a HIP runtime call or kernel launch failed */
+
+/* Element types of a logits tensor. */
+#define KA_DTYPE_BF16 0
+#define KA_DTYPE_F16 1
+#define KA_DTYPE_F32 2
+
+/* Library version string, e.g. "kernel_align_hip 0.1 (gfx950)". */
+const char *ka_version(void);
+/* Message of the last error on the calling thread ("" if none). */
+const char *ka_last_error(void);
+/* Name of a status code. */
+const char *ka_status_string(int status);
+
+/*
+ * Per-token log-probability:
+ *     out[r] = logits[r, ids[r]] - logsumexp_v(logits[r, :])          (fp32)
+ * for r in [0, n_rows).  logits is row-major [n_rows, vocab] with
+ * row_stride elements between rows; rows are the flattened G*L tokens.
+ * Replaces the chunk loop of SamplerBackend.compute_logp
+ * (rl_engine/kernels/sampling.py:92-112: log_softmax -> gather -> slice copy)
+ * and the native comparator (benchmarks/benchmark_grpo_op.py:52-54).
+ * One pass over the logits, fp32 accumulation, no temporary of the size of the
+ * logits.  A row's result depends on that row only and is reduced in a fixed
+ * order, so outputs are bit-identical across runs, batch sizes and chunkings.
+ * An id outside [0, vocab) yields NaN for that row.
+ */
+int ka_logprob_bf16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                    const int64_t *ids, float *out, void *hip_stream);
+int ka_logprob_f16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                   const int64_t *ids, float *out, void *hip_stream);
+int ka_logprob_f32(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                   const int64_t *ids, float *out, void *hip_stream);
+
+/*
+ * Same pass as ka_logprob_*, which also returns the entropy of each row's
+ * softmax, entropy[r] = -sum_v p_v log p_v (fp32).  entropy may be null.
+ * No counterpart in the reference; GRPO-style losses consume both.
+ */
+int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                            const int64_t *ids, float *out, float *entropy, void *hip_stream);
+
+/*
+ * Fused temperature -> top-k -> top-p -> draw, one token id per row.
+ * Replaces SamplerBackend.sample (rl_engine/kernels/sampling.py:39-88) with the
+ * filter semantics of native_sampling (benchmarks/benchmark_sampling.py:12-37):
+ *   1. if temperature != 1: y = logits / temperature, rounded to the logits dtype;
+ *   2. top_k > 0: keep {y >= k-th largest y}, ties included (top_k == 0: off);
+ *   3. top_p < 1: order kept entries by (y descending, index ascending), take
+ *      softmax over them, keep an entry iff the mass strictly before it is
+ *      <= top_p (the first entry crossing top_p stays); top_p == 1: off;
+ *   4. draw: over the survivors in ascending index order, pick the first index
+ *      whose inclusive cumulative mass exceeds uniforms[r] * total mass.
+ * Masses are exp(y - max y) evaluated by a fixed polynomial and truncated to
+ * 2^-40 fixed point, then summed as integers, so the result does not depend on
+ * summation order, batch size or launch geometry.
+ * uniforms: one fp32 in [0,1) per row.  out_ids: int64 [batch].
+ */
+size_t ka_sample_workspace_bytes(int64_t batch, int64_t vocab);
+int ka_sample_topk_topp_bf16(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                             float temperature, int32_t top_k, float top_p, const float *uniforms,
+                             int64_t *out_ids, void *workspace, size_t workspace_bytes,
+                             void *hip_stream);
+int ka_sample_topk_topp_f16(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                            float temperature, int32_t top_k, float top_p, const float *uniforms,
+                            int64_t *out_ids, void *workspace, size_t workspace_bytes,
+                            void *hip_stream);
+int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                            float temperature, int32_t top_k, float top_p, const float *uniforms,
+                            int64_t *out_ids, void *workspace, size_t workspace_bytes,
+                            void *hip_stream);
+
+/*
+ * Fused lm_head -> logprob without materialised logits:
+ *     out[r] = h_r . W[ids[r]] - logsumexp_v(h_r . W[v])               (fp32)
+ * hidden: bf16 [n_rows, hidden_dim] row-major; weight: bf16 [vocab, hidden_dim]
+ * row-major (the nn.Linear.weight layout).  bf16 MFMA with fp32 accumulation;
+ * logit tiles stay in registers and feed an online max / log-sum-exp.
+ * No counterpart in the reference; the nearest behaviour is
+ * compute_logp(lm_head(hidden)) (rl_engine/kernels/sampling.py:92-112).
+ */
+size_t ka_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab);
+int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                           int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
+                           size_t workspace_bytes, void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KERNEL_ALIGN_HIP_H */

@@ -1,0 +1,208 @@
+// Per-token logprob: out[r] = logits[r, ids[r]] - logsumexp(logits[r, :]).
+//
+// One workgroup owns one row.  Every lane streams 16-byte vectors of the row
+// (lane t takes vectors t, t + THREADS, ...) and keeps an online
+// (max, sum of 2^(x*log2e - max*log2e)) pair in fp32; the row is read exactly
+// once and nothing of the size of the logits is written.  The max is refreshed
+// once per group of UNROLL vectors, so the rescale costs one extra exp2 per
+// 8*UNROLL elements.  Lanes are combined by a fixed butterfly inside each
+// wavefront and then in wavefront order through LDS: a row's bits depend on
+// that row alone, never on the batch size, the chunking or the grid.
+#include "ka_common.h"
+
+namespace ka {
+namespace {
+
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr double kLn2 = 0.693147180559945309417232;
+// Running maxima start here instead of -inf so that (old max - new max) is
+// never inf - inf; logits below this are treated as -inf.
+constexpr float kFloor = -1.0e30f;
+
+struct RowState {
+    float m;    // running max of the lane's logits (>= kFloor)
+    float ml2;  // m * log2(e)
+    float s;    // sum of 2^(x*log2e - ml2)
+    float a;    // sum of x * 2^(x*log2e - ml2)   (entropy variant only)
+};
+
+template <int N, bool ENTROPY>
+__device__ __forceinline__ void fold(RowState &st, const float (&x)[N]) {
+    float mn = st.m;
+#pragma unroll
+    for (int j = 0; j < N; ++j) mn = fmaxf(mn, x[j]);
+    const float ml2n = mn * kLog2e;
+    const float rescale = fast_exp2(st.ml2 - ml2n);
+    float e[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) e[j] = fast_exp2(fmaf(x[j], kLog2e, -ml2n));
+    if (ENTROPY) {
+        float w[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) w[j] = (e[j] == 0.0f) ? 0.0f : x[j] * e[j];  // 0 * -inf stays 0
+#pragma unroll
+        for (int step = 1; step < N; step <<= 1)
+#pragma unroll
+            for (int j = 0; j + step < N; j += 2 * step) w[j] += w[j + step];
+        st.a = fmaf(st.a, rescale, w[0]);
+    }
+    // Pairwise tree in a fixed order.
+#pragma unroll
+    for (int step = 1; step < N; step <<= 1)
+#pragma unroll
+        for (int j = 0; j + step < N; j += 2 * step) e[j] += e[j + step];
+    st.s = fmaf(st.s, rescale, e[0]);
+    st.m = mn;
+    st.ml2 = ml2n;
+}
+
+template <typename T, int THREADS, int UNROLL, bool VEC, bool ENTROPY>
+__global__ __launch_bounds__(THREADS) void logprob_rows(const typename T::raw_t *__restrict__ logits,
+                                                        int64_t n_rows, int vocab, int64_t row_stride,
+                                                        const int64_t *__restrict__ ids,
+                                                        float *__restrict__ out,
+                                                        float *__restrict__ entropy) {
+    constexpr int EPV = T::kPerVec;
+    constexpr int NWAVES = THREADS / kWave;
+    __shared__ float red_a[NWAVES];
+    __shared__ float red_b[NWAVES];
+    __shared__ float red_c[NWAVES];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+
+    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        const typename T::raw_t *rp = logits + row * row_stride;
+
+        // Lane 0 fetches the target logit up front; its latency hides behind the stream.
+        float xt = __builtin_nanf("");
+        if (tid == 0) {
+            const int64_t id = ids[row];
+            if (id >= 0 && id < vocab) xt = T::widen(rp[id]);
+        }
+
+        RowState st{kFloor, kFloor * kLog2e, 0.0f, 0.0f};
+
+        if (VEC) {
+            const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+            const int nvec = vocab / EPV;
+            int i = tid;
+            for (; i + (UNROLL - 1) * THREADS < nvec; i += UNROLL * THREADS) {
+                uint4 v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) v[u] = load_stream(vp + i + u * THREADS);
+                float x[UNROLL * EPV];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    float xv[EPV];
+                    T::unpack(v[u], xv);
+#pragma unroll
+                    for (int j = 0; j < EPV; ++j) x[u * EPV + j] = xv[j];
+                }
+                fold<UNROLL * EPV, ENTROPY>(st, x);
+            }
+            for (; i < nvec; i += THREADS) {
+                float xv[EPV];
+                T::unpack(load_stream(vp + i), xv);
+                fold<EPV, ENTROPY>(st, xv);
+            }
+            const int tail = vocab - nvec * EPV;
+            if (tid < tail) {
+                const float xs[1] = {T::widen(rp[nvec * EPV + tid])};
+                fold<1, ENTROPY>(st, xs);
+            }
+        } else {
+            for (int i = tid; i < vocab; i += THREADS) {
+                const float xs[1] = {T::widen(rp[i])};
+                fold<1, ENTROPY>(st, xs);
+            }
+        }
+
+        // Row max (exact, order-free), then every lane's sum rebased to it.
+        const float wm = wave_max(st.ml2);
+        if (lane == 0) red_a[wave] = wm;
+        __syncthreads();
+        float big = red_a[0];
+#pragma unroll
+        for (int w = 1; w < NWAVES; ++w) big = fmaxf(big, red_a[w]);
+        const float rebase = fast_exp2(st.ml2 - big);
+        const float ws = wave_sum(st.s * rebase);
+        float wa = 0.0f;
+        if (ENTROPY) wa = wave_sum(st.a * rebase);
+        if (lane == 0) {
+            red_b[wave] = ws;
+            if (ENTROPY) red_c[wave] = wa;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float total = red_b[0];
+#pragma unroll
+            for (int w = 1; w < NWAVES; ++w) total += red_b[w];
+            const double lse = (double(big) + log2(double(total))) * kLn2;
+            out[row] = float(double(xt) - lse);
+            if (ENTROPY && entropy != nullptr) {
+                float ta = red_c[0];
+#pragma unroll
+                for (int w = 1; w < NWAVES; ++w) ta += red_c[w];
+                entropy[row] = float(lse - double(ta) / double(total));
+            }
+        }
+        // red_a / red_b are rewritten only after the next row's first barrier pair.
+        __syncthreads();
+    }
+}
+
+template <typename T, bool ENTROPY>
+int launch(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride, const int64_t *ids,
+           float *out, float *entropy, void *hip_stream) {
+    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "logprob: n_rows %lld < 0", (long long)n_rows);
+    if (n_rows == 0) return KA_OK;
+    if (logits == nullptr || ids == nullptr || out == nullptr)
+        return fail(KA_ERR_BAD_ARG, "logprob: null logits / ids / out pointer");
+    if (vocab < 1) return fail(KA_ERR_BAD_ARG, "logprob: vocab %lld < 1", (long long)vocab);
+    if (vocab >= (int64_t(1) << 31))
+        return fail(KA_ERR_UNSUPPORTED, "logprob: vocab %lld does not fit 31 bits", (long long)vocab);
+    if (row_stride < vocab)
+        return fail(KA_ERR_BAD_ARG, "logprob: row_stride %lld < vocab %lld", (long long)row_stride,
+                    (long long)vocab);
+
+    constexpr int THREADS = 256;
+    constexpr int UNROLL = 4;
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const auto *lp = static_cast<const typename T::raw_t *>(logits);
+    const bool aligned = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) &&
+                         ((row_stride * T::kBytes) % 16 == 0);
+    const unsigned grid = unsigned(n_rows < (int64_t(1) << 30) ? n_rows : (int64_t(1) << 30));
+    if (aligned) {
+        hipLaunchKernelGGL((logprob_rows<T, THREADS, UNROLL, true, ENTROPY>), dim3(grid), dim3(THREADS), 0,
+                           stream, lp, n_rows, int(vocab), row_stride, ids, out, entropy);
+    } else {
+        hipLaunchKernelGGL((logprob_rows<T, THREADS, 1, false, ENTROPY>), dim3(grid), dim3(THREADS), 0,
+                           stream, lp, n_rows, int(vocab), row_stride, ids, out, entropy);
+    }
+    return check_hip(hipGetLastError(), "logprob launch");
+}
+
+}  // namespace
+}  // namespace ka
+
+KA_EXPORT int ka_logprob_bf16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                              const int64_t *ids, float *out, void *hip_stream) {
+    return ka::launch<ka::Bf16, false>(logits, n_rows, vocab, row_stride, ids, out, nullptr, hip_stream);
+}
+
+KA_EXPORT int ka_logprob_f16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                             const int64_t *ids, float *out, void *hip_stream) {
+    return ka::launch<ka::F16, false>(logits, n_rows, vocab, row_stride, ids, out, nullptr, hip_stream);
+}
+
+KA_EXPORT int ka_logprob_f32(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                             const int64_t *ids, float *out, void *hip_stream) {
+    return ka::launch<ka::F32, false>(logits, n_rows, vocab, row_stride, ids, out, nullptr, hip_stream);
+}
+
+KA_EXPORT int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_t vocab,
+                                      int64_t row_stride, const int64_t *ids, float *out,
+                                      float *entropy, void *hip_stream) {
+    return ka::launch<ka::Bf16, true>(logits, n_rows, vocab, row_stride, ids, out, entropy, hip_stream);
+}

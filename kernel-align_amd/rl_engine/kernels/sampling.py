@@ -1,0 +1,213 @@
+"""SamplerBackend: the logprob and sampling operators on hand-written gfx950 kernels.
+
+Drop-in for the reference's rl_engine/kernels/sampling.py:9-112: a parameter-less
+nn.Module with ``compute_logp(logits, token_ids)`` and
+``sample(logits, top_k, top_p, temperature, deterministic)``.  Every call goes
+to libkernel_align_hip.so on the current HIP stream; nothing runs on the CPU and
+nothing falls back to torch ops.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from rl_engine.kernels import _hip
+from rl_engine.kernels.pool import WorkspacePool
+from rl_engine.platforms.constants import constants
+from rl_engine.utils.logger import logger
+
+# Rows (tokens) per kernel launch of compute_logp.  The kernel keeps no
+# per-launch state, so this is launch granularity only: it bounds how long one
+# launch occupies the GPU and never changes a result bit.
+DEFAULT_CHUNK_TOKENS = 8192
+
+_LOGPROB_FN = {torch.bfloat16: "ka_logprob_bf16", torch.float16: "ka_logprob_f16",
+               torch.float32: "ka_logprob_f32"}
+_SAMPLE_FN = {torch.bfloat16: "ka_sample_topk_topp_bf16", torch.float16: "ka_sample_topk_topp_f16",
+              torch.float32: "ka_sample_topk_topp_f32"}
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU: rl_engine has no CPU path (got {t.device})")
+
+
+def _rows_view(logits: torch.Tensor) -> torch.Tensor:
+    """[.., V] -> [N, V] with unit stride along V and a uniform row stride, copying only if needed."""
+    vocab = logits.shape[-1]
+    if logits.dim() == 2 and logits.stride(1) == 1 and (logits.shape[0] <= 1 or logits.stride(0) >= vocab):
+        return logits
+    if logits.is_contiguous():
+        return logits.view(-1, vocab)
+    logger.warn_once("logits are not row-contiguous: copying them before the kernel launch")
+    return logits.contiguous().view(-1, vocab)
+
+
+class SamplerBackend(nn.Module):
+    def __init__(self, pool_bytes: int | None = None):
+        super().__init__()
+        self.backend = self._detect_backend()
+        self._init_backend_assets(pool_bytes)
+
+    def _detect_backend(self) -> str:
+        logger.info_once("AMD GPU (ROCm): using the in-tree HIP kernels")
+        return constants.BackendLib.HIP_NATIVE.value
+
+    def _init_backend_assets(self, pool_bytes: int | None) -> None:
+        # Loading here makes a missing or incomplete library fail at construction.
+        self._lib = _hip.load()
+        self.pool = WorkspacePool(pool_bytes)
+        logger.info_once(f"Loaded {self._lib.ka_version().decode()}")
+
+    # ------------------------------------------------------------------ logprob
+    @torch.inference_mode()
+    def compute_logp(self, logits, token_ids, out_dtype=torch.float32, chunk_tokens=None):
+        """Per-token log-probabilities ``log_softmax(logits, -1)[..., token_ids]``.
+
+        logits: [G, L, V] (or [N, V]) bf16 / fp16 / fp32 on the GPU; token_ids: integer tensor of
+        shape logits.shape[:-1].  Returns fp32 of shape [G, L] (reference:
+        sampling.py:92-112 returns logits.dtype; pass ``out_dtype=logits.dtype`` for that).
+        The rows are fed to the kernel ``chunk_tokens`` at a time; no chunk-sized buffer exists.
+        """
+        _require_gpu(logits, "logits")
+        if logits.dim() < 2:
+            raise ValueError("logits must be [..., V]")
+        if tuple(token_ids.shape) != tuple(logits.shape[:-1]):
+            raise ValueError(f"token_ids shape {tuple(token_ids.shape)} != logits.shape[:-1] "
+                             f"{tuple(logits.shape[:-1])}")
+        fn_name = _LOGPROB_FN.get(logits.dtype)
+        if fn_name is None:
+            raise TypeError(f"unsupported logits dtype {logits.dtype}")
+        fn = getattr(self._lib, fn_name)
+        rows = _rows_view(logits)
+        n_rows, vocab = rows.shape
+        ids = token_ids.to(device=logits.device, dtype=torch.int64).contiguous().view(-1)
+        out = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
+        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
+        if chunk < 1:
+            raise ValueError("chunk_tokens must be >= 1")
+        row_stride = rows.stride(0) if n_rows > 1 else vocab
+        esize = rows.element_size()
+        with torch.cuda.device(logits.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            base, ids_base, out_base = rows.data_ptr(), ids.data_ptr(), out.data_ptr()
+            for start in range(0, n_rows, chunk):
+                n = min(chunk, n_rows - start)
+                status = fn(base + start * row_stride * esize, n, vocab, row_stride,
+                            ids_base + start * 8, out_base + start * 4, stream)
+                _hip.check(status, fn_name)
+        if out_dtype != torch.float32:
+            out = out.to(out_dtype)
+        return out.view(tuple(logits.shape[:-1]))
+
+    @torch.inference_mode()
+    def compute_logp_entropy(self, logits, token_ids, chunk_tokens=None):
+        """compute_logp plus the entropy of every row's softmax, from the same single pass (bf16)."""
+        _require_gpu(logits, "logits")
+        if logits.dtype != torch.bfloat16:
+            raise TypeError("compute_logp_entropy takes bf16 logits")
+        if tuple(token_ids.shape) != tuple(logits.shape[:-1]):
+            raise ValueError("token_ids shape must equal logits.shape[:-1]")
+        rows = _rows_view(logits)
+        n_rows, vocab = rows.shape
+        ids = token_ids.to(device=logits.device, dtype=torch.int64).contiguous().view(-1)
+        out = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
+        ent = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
+        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
+        row_stride = rows.stride(0) if n_rows > 1 else vocab
+        with torch.cuda.device(logits.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            for start in range(0, n_rows, chunk):
+                n = min(chunk, n_rows - start)
+                status = self._lib.ka_logprob_entropy_bf16(
+                    rows.data_ptr() + start * row_stride * 2, n, vocab, row_stride,
+                    ids.data_ptr() + start * 8, out.data_ptr() + start * 4, ent.data_ptr() + start * 4, stream)
+                _hip.check(status, "ka_logprob_entropy_bf16")
+        shape = tuple(logits.shape[:-1])
+        return out.view(shape), ent.view(shape)
+
+    # ----------------------------------------------------------------- sampling
+    @torch.inference_mode()
+    def sample(self, logits, top_k=None, top_p=None, temperature=1.0, deterministic=True,
+               uniforms=None, generator=None):
+        """Draw one token id per row after temperature -> top-k -> top-p filtering.
+
+        logits: [B, V] bf16 / fp16 / fp32 on the GPU.  Returns int64 [B] (reference:
+        sampling.py:39-88; filter semantics of benchmarks/benchmark_sampling.py:12-37).
+        ``uniforms`` ([B] fp32 in [0, 1)) drives the draw; if None they come from
+        ``torch.rand(B, generator=generator)`` on the logits' device.  The kernels are always
+        deterministic, so ``deterministic`` is accepted and ignored.
+        """
+        _require_gpu(logits, "logits")
+        if logits.dim() != 2:
+            raise ValueError("logits must be [B, V]")
+        fn_name = _SAMPLE_FN.get(logits.dtype)
+        if fn_name is None:
+            raise TypeError(f"unsupported logits dtype {logits.dtype}")
+        batch, vocab = logits.shape
+        k = 0 if top_k is None else int(top_k)
+        if top_k is not None and k < 1:
+            raise ValueError(f"top_k must be >= 1 (got {top_k})")
+        p = 1.0 if top_p is None else float(top_p)
+        if not 0.0 < p <= 1.0:
+            raise ValueError(f"top_p must be in (0, 1] (got {top_p})")
+        temperature = float(temperature)
+        if not temperature > 0.0:
+            raise ValueError(f"temperature must be > 0 (got {temperature})")
+        rows = _rows_view(logits)
+        if uniforms is None:
+            uniforms = torch.rand(batch, generator=generator, device=logits.device, dtype=torch.float32)
+        else:
+            if tuple(uniforms.shape) != (batch,):
+                raise ValueError(f"uniforms must have shape ({batch},)")
+            uniforms = uniforms.to(device=logits.device, dtype=torch.float32).contiguous()
+        out = torch.empty(batch, dtype=torch.int64, device=logits.device)
+        if batch == 0:
+            return out
+        ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
+        self.pool.reset()
+        ws = self.pool.reserve(ws_bytes, logits.device)
+        row_stride = rows.stride(0) if batch > 1 else vocab
+        with torch.cuda.device(logits.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            status = getattr(self._lib, fn_name)(
+                rows.data_ptr(), batch, vocab, row_stride, temperature, k, p, uniforms.data_ptr(),
+                out.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+        _hip.check(status, fn_name)
+        return out
+
+    # ---------------------------------------------------------------- fused GEMM
+    @torch.inference_mode()
+    def fused_linear_logp(self, hidden, weight, token_ids):
+        """``compute_logp(hidden @ weight.T, token_ids)`` without materialising the logits.
+
+        hidden: bf16 [..., H]; weight: bf16 [V, H] (nn.Linear.weight layout); token_ids: integer
+        tensor of shape hidden.shape[:-1].  Returns fp32 of that shape.
+        """
+        _require_gpu(hidden, "hidden")
+        _require_gpu(weight, "weight")
+        if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            raise TypeError("fused_linear_logp takes bf16 hidden and weight")
+        if weight.dim() != 2 or hidden.shape[-1] != weight.shape[1]:
+            raise ValueError("weight must be [V, H] with H == hidden.shape[-1]")
+        if tuple(token_ids.shape) != tuple(hidden.shape[:-1]):
+            raise ValueError("token_ids shape must equal hidden.shape[:-1]")
+        hdim = hidden.shape[-1]
+        vocab = weight.shape[0]
+        h2 = hidden.contiguous().view(-1, hdim)
+        w2 = weight.contiguous()
+        n_rows = h2.shape[0]
+        ids = token_ids.to(device=hidden.device, dtype=torch.int64).contiguous().view(-1)
+        out = torch.empty(n_rows, dtype=torch.float32, device=hidden.device)
+        if n_rows == 0:
+            return out.view(tuple(hidden.shape[:-1]))
+        ws_bytes = self._lib.ka_lmhead_workspace_bytes(n_rows, hdim, vocab)
+        self.pool.reset()
+        ws = self.pool.reserve(ws_bytes, hidden.device)
+        with torch.cuda.device(hidden.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            status = self._lib.ka_lmhead_logprob_bf16(
+                h2.data_ptr(), w2.data_ptr(), ids.data_ptr(), out.data_ptr(), n_rows, hdim, vocab,
+                ws.data_ptr(), ws_bytes, stream)
+        _hip.check(status, "ka_lmhead_logprob_bf16")
+        return out.view(tuple(hidden.shape[:-1]))

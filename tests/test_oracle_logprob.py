@@ -1,0 +1,97 @@
+"""Pins oracle/logprob_ref.py: closed forms, brute force and fp32-vs-fp64 agreement (CPU only)."""
+import math
+
+import pytest
+import torch
+
+from oracle import logprob_ref as O
+
+
+def test_uniform_row_is_minus_log_v():
+    for v in (2, 17, 1000, 32000):
+        x = torch.full((1, v), 3.25, dtype=torch.bfloat16)
+        ids = torch.tensor([v // 2])
+        assert abs(O.logprob_ref(x, ids).item() + math.log(v)) < 2e-6 * max(1, math.log(v))
+        assert abs(O.logprob_f64(x, ids).item() + math.log(v)) < 1e-12
+
+
+def test_single_spike_closed_form():
+    v, c = 128256, 25.0
+    x = torch.zeros(2, v, dtype=torch.bfloat16)
+    x[:, 777] = c
+    ids = torch.tensor([777, 5])
+    lse_minus_c = math.log1p((v - 1) * math.exp(-c))
+    want = [-lse_minus_c, -c - lse_minus_c]
+    got32, got64 = O.logprob_ref(x, ids), O.logprob_f64(x, ids)
+    for k in range(2):
+        assert abs(got64[k].item() - want[k]) < 1e-12
+        assert abs(got32[k].item() - want[k]) < 1e-5
+
+
+def test_masked_entries_contribute_nothing():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4, 64, generator=g).bfloat16()
+    ids = torch.randint(0, 32, (4,), generator=g)
+    masked = torch.cat([x[:, :32], torch.full((4, 32), -math.inf, dtype=torch.bfloat16)], dim=1)
+    assert torch.equal(O.logprob_ref(masked, ids), O.logprob_ref(x[:, :32].contiguous(), ids))
+    assert torch.allclose(O.logprob_f64(masked, ids), O.logprob_f64(x[:, :32].contiguous(), ids), atol=1e-14)
+
+
+def test_probabilities_sum_to_one():
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(1, 501, generator=g) * 3).bfloat16()
+    all_targets = torch.arange(501)
+    rows = x.expand(501, 501)
+    assert abs(O.logprob_f64(rows, all_targets).exp().sum().item() - 1.0) < 1e-12
+    assert abs(O.logprob_ref(rows, all_targets).double().exp().sum().item() - 1.0) < 1e-5
+
+
+def test_shift_invariance_with_exact_shift():
+    # adding 8.0 keeps every bf16 value in [-4, 4) with <= 4 mantissa bits exactly representable
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randint(-32, 32, (3, 300), generator=g).float() / 8).bfloat16()
+    ids = torch.randint(0, 300, (3,), generator=g)
+    shifted = (x.float() + 8.0).bfloat16()
+    assert torch.equal(shifted.float() - 8.0, x.float())
+    assert torch.allclose(O.logprob_f64(x, ids), O.logprob_f64(shifted, ids), atol=1e-13)
+    assert torch.allclose(O.logprob_ref(x, ids), O.logprob_ref(shifted, ids), atol=2e-6)
+
+
+@pytest.mark.parametrize("vocab", [1, 2, 7, 64])
+def test_bruteforce_small_vocab(vocab):
+    g = torch.Generator().manual_seed(vocab)
+    x = (torch.randn(5, vocab, generator=g) * 4).bfloat16()
+    ids = torch.randint(0, vocab, (5,), generator=g)
+    got64, got32 = O.logprob_f64(x, ids), O.logprob_ref(x, ids)
+    for r in range(5):
+        want = O.logprob_bruteforce(x[r].float().tolist(), int(ids[r]))
+        assert abs(got64[r].item() - want) < 1e-12
+        assert abs(got32[r].item() - want) < 2e-6
+
+
+def test_fp32_route_within_tolerance_of_fp64_on_cfg1():
+    from benchmarks.workloads import cfg1_logits
+
+    logits, ids = cfg1_logits()
+    a, b = O.logprob_ref(logits, ids), O.logprob_f64(logits, ids)
+    assert a.shape == (4, 128) and a.dtype == torch.float32
+    assert (a.double() - b).abs().max().item() < 2e-5
+
+
+def test_reference_dtype_route_is_the_rounded_one():
+    # what the reference returns on ROCm (bf16) is far from the fp32 value: it cannot be the oracle
+    from benchmarks.workloads import cfg1_logits
+
+    logits, ids = cfg1_logits()
+    ref_bf16 = O.logprob_reference_dtype(logits[:1], ids[:1])
+    assert ref_bf16.dtype == torch.bfloat16
+    err = (ref_bf16.double() - O.logprob_f64(logits[:1], ids[:1])).abs().max().item()
+    assert 1e-3 < err < 0.25
+
+
+def test_entropy_closed_forms():
+    v = 4096
+    assert abs(O.entropy_f64(torch.zeros(1, v, dtype=torch.bfloat16)).item() - math.log(v)) < 1e-12
+    x = torch.full((1, v), -math.inf, dtype=torch.bfloat16)
+    x[0, 3] = 1.0
+    assert O.entropy_f64(x).item() == 0.0
