@@ -66,6 +66,9 @@ def main() -> int:
     ap.add_argument("--cpu-sample-rows", type=int, default=32768,
                     help="rows of the tensor the CPU oracle is timed on (0 = skip)")
     ap.add_argument("--chunk-tokens", type=int, default=None, help="rows per kernel launch")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (torch copy_) three times, so a counter "
+                         "run of this command holds a kernel of known traffic to scale FETCH/WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         log(f"bench.py measures one GPU: --gpus {args.gpus} is not supported in this build "
@@ -90,6 +93,14 @@ def main() -> int:
     logits, ids = spike_logits(n_rows, V, seed=0, device=dev)
     logits3, ids2 = logits.view(G, L, V), ids.view(G, L)
     torch.cuda.synchronize()
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         sampler.compute_logp(logits3, ids2, chunk_tokens=chunk)
