@@ -1,13 +1,488 @@
-// Fused sampling (placeholder entry points while the kernels are being written).
+// Fused temperature -> top-k -> top-p -> draw, one workgroup per row.
+//
+// Every decision is taken on integers, so the sampled id does not depend on
+// summation order, batch size or launch geometry:
+//   * each scaled logit y maps to an order-preserving 32-bit key;
+//   * the k-th largest key K* comes from an MSB-first radix descent over
+//     2048-bin LDS count histograms (ties with K* survive, as in the reference);
+//   * softmax masses are W(y - max) = trunc(2^40 * exp(y - max)), evaluated by a
+//     fixed sequence of IEEE double operations, and summed as 64-bit integers;
+//   * the top-p cut is a second radix descent over per-bin integer mass: it finds
+//     the lowest key Kc whose first entry still has (mass before it) <= top_p * Z,
+//     and how many entries r of the Kc tie group (ascending index) survive;
+//   * the draw walks the row once more in index order with block-wide integer
+//     prefix sums and stops at the first survivor whose inclusive mass exceeds
+//     floor(u * Z_survivors).
+// The row is re-read by every pass; after the first it comes from L2 / MALL.
 #include "ka_common.h"
 
-KA_EXPORT size_t ka_sample_workspace_bytes(int64_t batch, int64_t vocab) { return 256; }
+namespace ka {
+namespace {
 
-#define KA_SAMPLE_STUB(name)                                                                          \
-    KA_EXPORT int name(const void *, int64_t, int64_t, int64_t, float, int32_t, float, const float *, \
-                       int64_t *, void *, size_t, void *) {                                           \
-        return ka::fail(KA_ERR_UNSUPPORTED, #name ": not implemented");                               \
+constexpr int S_THREADS = 1024;
+constexpr int S_WAVES = S_THREADS / kWave;
+constexpr int BINS = 2048;
+constexpr int FIX_BITS = 40;
+
+// ---------------------------------------------------------------------------
+// Scalar helpers (all exact)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t key_of(float y) {
+    const uint32_t b = __float_as_uint(y);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float value_of(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// W(d) = trunc(2^40 * exp(d)), d <= 0.  Separate IEEE multiplies and adds (the
+// _rn intrinsics are never contracted into FMAs), Taylor coefficients 1/k!.
+__device__ __forceinline__ uint64_t weight_fix(float d) {
+    constexpr double C[12] = {0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,
+                              0x1.5555555555555p-3,  0x1.5555555555555p-5,  0x1.1111111111111p-7,
+                              0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16,
+                              0x1.71de3a556c734p-19, 0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26};
+    constexpr double LOG2E = 0x1.71547652b82fep+0, LN2 = 0x1.62e42fefa39efp-1;
+    if (!(d <= 0.0f)) return d > 0.0f ? (uint64_t(1) << FIX_BITS) : 0;
+    const double t = __dmul_rn(double(d), LOG2E);
+    if (t < -41.0) return 0;
+    const int n = int(__dadd_rn(t, -0.5));
+    const double f = __dsub_rn(t, double(n));
+    const double g = __dmul_rn(f, LN2);
+    double p = C[11];
+#pragma unroll
+    for (int k = 10; k >= 0; --k) {
+        p = __dmul_rn(p, g);
+        p = __dadd_rn(p, C[k]);
     }
-KA_SAMPLE_STUB(ka_sample_topk_topp_bf16)
-KA_SAMPLE_STUB(ka_sample_topk_topp_f16)
-KA_SAMPLE_STUB(ka_sample_topk_topp_f32)
+    const double scale = __longlong_as_double((long long)(uint64_t(1023 + FIX_BITS + n) << 52));
+    return (uint64_t)__dmul_rn(p, scale);
+}
+
+// floor(s * z) for an fp32 0 <= s < 1 and z < 2^62.
+__device__ __forceinline__ uint64_t floor_scale(float s, uint64_t z) {
+    const uint32_t b = __float_as_uint(s);
+    const uint32_t e = (b >> 23) & 0xffu, m = b & 0x7fffffu;
+    if (e == 0 && m == 0) return 0;
+    uint64_t mant;
+    int shift;
+    if (e == 0) { mant = m; shift = 149; } else { mant = m | 0x800000u; shift = 150 - int(e); }
+    const uint64_t lo = mant * z, hi = __umul64hi(mant, z);
+    if (shift >= 128) return 0;
+    if (shift >= 64) return hi >> (shift - 64);
+    return (lo >> shift) | (hi << (64 - shift));  // 24 <= shift < 64
+}
+
+// y = x / T rounded to the logits dtype (torch's `logits / temperature`), -0 folded to +0.
+template <typename T> struct Round;
+template <> struct Round<Bf16> {
+    static __device__ __forceinline__ float apply(float q) {
+        uint32_t b = __float_as_uint(q);
+        if ((b & 0x7fffffffu) > 0x7f800000u) return __uint_as_float(((b >> 16) | 0x40u) << 16);
+        b += 0x7fffu + ((b >> 16) & 1u);
+        return __uint_as_float(b & 0xffff0000u);
+    }
+    static constexpr int kLevels = 2;
+};
+template <> struct Round<F16> {
+    static __device__ __forceinline__ float apply(float q) { return float(_Float16(q)); }
+    static constexpr int kLevels = 2;
+};
+template <> struct Round<F32> {
+    static __device__ __forceinline__ float apply(float q) { return q; }
+    static constexpr int kLevels = 3;
+};
+
+// Radix levels, most significant first.  A widened bf16 occupies the top 16 key bits
+// (1 + 8 + 7), a widened fp16 the top 19 (1 + 8 + 10), fp32 all 32.
+template <typename T> __device__ __forceinline__ int level_shift(int level) {
+    if (T::kDtype == KA_DTYPE_BF16) return level == 0 ? 21 : 16;
+    if (T::kDtype == KA_DTYPE_F16) return level == 0 ? 21 : 13;
+    return level == 0 ? 21 : (level == 1 ? 10 : 0);
+}
+template <typename T> __device__ __forceinline__ int level_bits(int level) {
+    if (T::kDtype == KA_DTYPE_BF16) return level == 0 ? 11 : 5;
+    if (T::kDtype == KA_DTYPE_F16) return level == 0 ? 11 : 8;
+    return level == 2 ? 10 : 11;
+}
+
+template <typename T>
+__device__ __forceinline__ uint32_t elem_key(typename T::raw_t raw, float temp, bool has_t) {
+    float y = T::widen(raw);
+    if (has_t) y = Round<T>::apply(y / temp);
+    y = (y == 0.0f) ? 0.0f : y;
+    return key_of(y);
+}
+
+// ---------------------------------------------------------------------------
+// Block-wide primitives (1024 threads, fixed exchange pattern)
+// ---------------------------------------------------------------------------
+struct Shared {
+    uint32_t cnt[BINS];
+    uint64_t mass[BINS];
+    uint64_t wave_u64[S_WAVES];
+    uint32_t wave_u32[S_WAVES];
+    // broadcast slots
+    uint32_t sel_digit, sel_above, sel_count;
+    uint64_t sel_mass_above, sel_mass;
+    int best_rb;
+    uint32_t max_key;
+    int64_t hit;
+};
+
+template <typename V> __device__ __forceinline__ V shfl_up_v(V v, int off) { return __shfl_up(v, off, kWave); }
+
+// Exclusive prefix sum over the block in thread order; *total = block sum.  Contains barriers.
+template <typename V>
+__device__ __forceinline__ V block_excl_scan(V v, V *wave_buf, V *total) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    V inc = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const V t = shfl_up_v(inc, off);
+        if (lane >= off) inc += t;
+    }
+    __syncthreads();  // wave_buf may still be read from a previous call
+    if (lane == kWave - 1) wave_buf[wave] = inc;
+    __syncthreads();
+    V base = 0, sum = 0;
+#pragma unroll
+    for (int w = 0; w < S_WAVES; ++w) {
+        const V x = wave_buf[w];
+        if (w < wave) base += x;
+        sum += x;
+    }
+    *total = sum;
+    return base + inc - v;
+}
+
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, Shared &sh) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t t = __shfl_xor(v, off, kWave);
+        v = t > v ? t : v;
+    }
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) sh.wave_u32[threadIdx.x / kWave] = v;
+    __syncthreads();
+    uint32_t r = sh.wave_u32[0];
+#pragma unroll
+    for (int w = 1; w < S_WAVES; ++w) r = sh.wave_u32[w] > r ? sh.wave_u32[w] : r;
+    return r;
+}
+
+__device__ __forceinline__ void clear_hist(Shared &sh) {
+    for (int b = threadIdx.x; b < BINS; b += S_THREADS) {
+        sh.cnt[b] = 0;
+        sh.mass[b] = 0;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row traversal: f(index, key) for every element, any order.
+// ---------------------------------------------------------------------------
+template <typename T, typename F>
+__device__ __forceinline__ void for_each_key(const typename T::raw_t *rp, int vocab, bool vec, float temp,
+                                             bool has_t, F &&f) {
+    constexpr int EPV = T::kPerVec;
+    const int tid = threadIdx.x;
+    if (vec) {
+        const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+        const int nvec = vocab / EPV;
+        constexpr int U = 4;
+        int v = tid;
+        for (; v + (U - 1) * S_THREADS < nvec; v += U * S_THREADS) {
+            uint4 q[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) q[u] = vp[v + u * S_THREADS];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[u]);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) f((v + u * S_THREADS) * EPV + j, elem_key<T>(e[j], temp, has_t));
+            }
+        }
+        for (; v < nvec; v += S_THREADS) {
+            const uint4 q = vp[v];
+            const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) f(v * EPV + j, elem_key<T>(e[j], temp, has_t));
+        }
+        const int i = nvec * EPV + tid;
+        if (i < vocab) f(i, elem_key<T>(rp[i], temp, has_t));
+    } else {
+        for (int i = tid; i < vocab; i += S_THREADS) f(i, elem_key<T>(rp[i], temp, has_t));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The kernel
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t *__restrict__ logits,
+                                                         int vocab, int64_t row_stride, float temp,
+                                                         int top_k, float top_p,
+                                                         const float *__restrict__ uniforms,
+                                                         int64_t *__restrict__ out, int vec) {
+    constexpr int EPV = T::kPerVec;
+    constexpr int LEVELS = Round<T>::kLevels;
+    __shared__ Shared sh;
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const typename T::raw_t *rp = logits + row * row_stride;
+    const bool has_t = temp != 1.0f;
+    const bool use_k = top_k > 0 && top_k < vocab;
+    const bool use_p = top_p < 1.0f;
+
+    // ---- pass 0: row maximum and the level-0 count histogram --------------------------
+    clear_hist(sh);
+    __syncthreads();
+    uint32_t kmax = 0;
+    for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
+        kmax = key > kmax ? key : kmax;
+        if (use_k) atomicAdd(&sh.cnt[key >> 21], 1u);
+    });
+    kmax = block_max_u32(kmax, sh);  // barriers inside also publish the histogram
+    const float vmax = value_of(kmax);
+
+    // ---- top-k: MSB-first descent to the k-th largest key --------------------------------
+    uint32_t kstar = 0;      // keep key >= kstar
+    uint32_t n_eq_kstar = 0; // entries equal to kstar (only meaningful with use_k)
+    if (use_k) {
+        uint32_t rank = uint32_t(top_k);  // 1-based rank inside the current prefix
+        uint32_t prefix = 0;
+        for (int level = 0; level < LEVELS; ++level) {
+            const int shift = level_shift<T>(level), bits = level_bits<T>(level);
+            const uint32_t nb = 1u << bits;
+            if (level > 0) {
+                clear_hist(sh);
+                __syncthreads();
+                const int pshift = level_shift<T>(level - 1);
+                for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
+                    if ((key >> pshift) == prefix) atomicAdd(&sh.cnt[(key >> shift) & (nb - 1)], 1u);
+                });
+                __syncthreads();
+            }
+            // thread t owns the bins 2t and 2t+1 counted from the top
+            const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
+            const uint32_t c0 = rb0 < int(nb) ? sh.cnt[nb - 1 - rb0] : 0u;
+            const uint32_t c1 = rb1 < int(nb) ? sh.cnt[nb - 1 - rb1] : 0u;
+            uint32_t total;
+            const uint32_t excl = block_excl_scan<uint32_t>(c0 + c1, sh.wave_u32, &total);
+            if (excl < rank && rank <= excl + c0) {
+                sh.sel_digit = nb - 1 - rb0; sh.sel_above = excl; sh.sel_count = c0;
+            } else if (excl + c0 < rank && rank <= excl + c0 + c1) {
+                sh.sel_digit = nb - 1 - rb1; sh.sel_above = excl + c0; sh.sel_count = c1;
+            }
+            __syncthreads();
+            prefix = (prefix << bits) | sh.sel_digit;
+            rank -= sh.sel_above;
+            n_eq_kstar = sh.sel_count;
+            __syncthreads();
+        }
+        kstar = prefix << level_shift<T>(LEVELS - 1);
+    }
+
+    // ---- masses of the survivors of top-k: total, and level-0 histogram for top-p ---------
+    clear_hist(sh);
+    __syncthreads();
+    uint64_t zpart = 0;
+    for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
+        if (key >= kstar) {
+            const float y = value_of(key);
+            const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
+            zpart += w;
+            if (use_p) {
+                atomicAdd(reinterpret_cast<unsigned long long *>(&sh.mass[key >> 21]), (unsigned long long)w);
+                atomicAdd(&sh.cnt[key >> 21], 1u);
+            }
+        }
+    });
+    uint64_t z_topk;
+    block_excl_scan<uint64_t>(zpart, sh.wave_u64, &z_topk);
+    __syncthreads();
+
+    // ---- top-p: descent to the lowest key whose first entry is still kept ------------------
+    uint32_t kcut = kstar;            // survivors: key > kcut, or key == kcut with tie rank < r_cut
+    uint32_t r_cut = 0xffffffffu;
+    uint64_t z_kept = z_topk;
+    if (use_p) {
+        const uint64_t theta = floor_scale(top_p, z_topk);
+        uint64_t before = 0;          // mass of the keys above the current prefix
+        uint32_t prefix = 0;
+        uint32_t n_cut = 0;
+        uint64_t m_cut = 0;
+        for (int level = 0; level < LEVELS; ++level) {
+            const int shift = level_shift<T>(level), bits = level_bits<T>(level);
+            const uint32_t nb = 1u << bits;
+            if (level > 0) {
+                clear_hist(sh);
+                __syncthreads();
+                const int pshift = level_shift<T>(level - 1);
+                for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
+                    if (key >= kstar && (key >> pshift) == prefix) {
+                        const float y = value_of(key);
+                        const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
+                        const uint32_t d = (key >> shift) & (nb - 1);
+                        atomicAdd(reinterpret_cast<unsigned long long *>(&sh.mass[d]), (unsigned long long)w);
+                        atomicAdd(&sh.cnt[d], 1u);
+                    }
+                });
+                __syncthreads();
+            }
+            const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
+            const uint64_t m0 = rb0 < int(nb) ? sh.mass[nb - 1 - rb0] : 0ull;
+            const uint64_t m1 = rb1 < int(nb) ? sh.mass[nb - 1 - rb1] : 0ull;
+            const uint32_t c0 = rb0 < int(nb) ? sh.cnt[nb - 1 - rb0] : 0u;
+            const uint32_t c1 = rb1 < int(nb) ? sh.cnt[nb - 1 - rb1] : 0u;
+            uint64_t total;
+            const uint64_t excl = block_excl_scan<uint64_t>(m0 + m1, sh.wave_u64, &total);
+            if (tid == 0) sh.best_rb = -1;
+            __syncthreads();
+            const bool q0 = c0 > 0 && before + excl <= theta;
+            const bool q1 = c1 > 0 && before + excl + m0 <= theta;
+            if (q1) atomicMax(&sh.best_rb, rb1);
+            else if (q0) atomicMax(&sh.best_rb, rb0);
+            __syncthreads();
+            const int best = sh.best_rb;
+            if (best == rb0) { sh.sel_mass_above = excl; sh.sel_mass = m0; sh.sel_count = c0; }
+            if (best == rb1) { sh.sel_mass_above = excl + m0; sh.sel_mass = m1; sh.sel_count = c1; }
+            __syncthreads();
+            prefix = (prefix << bits) | uint32_t(nb - 1 - best);
+            before += sh.sel_mass_above;
+            n_cut = sh.sel_count;
+            m_cut = sh.sel_mass;
+            __syncthreads();
+        }
+        kcut = prefix << level_shift<T>(LEVELS - 1);
+        const uint64_t w_cut = n_cut ? m_cut / n_cut : 0;   // every entry of the tie group has this mass
+        uint64_t r = n_cut;
+        if (w_cut > 0) {
+            const uint64_t fit = (theta - before) / w_cut + 1;  // entries t with before + t*w <= theta
+            r = fit < r ? fit : r;
+        }
+        r_cut = uint32_t(r);
+        z_kept = before + r * w_cut;
+        if (r == n_cut) r_cut = 0xffffffffu;  // whole tie group survives: no rank bookkeeping needed
+    }
+
+    // ---- draw: first survivor, in index order, whose inclusive mass exceeds floor(u * Z) ----
+    float u = uniforms[row];
+    if (!(u >= 0.0f)) u = 0.0f;
+    if (u >= 1.0f) u = __uint_as_float(0x3f7fffffu);
+    const uint64_t tau = floor_scale(u, z_kept);
+    const bool track_ties = r_cut != 0xffffffffu;
+    if (tid == 0) sh.hit = -1;
+    uint64_t carry_mass = 0;
+    uint32_t carry_ties = 0;
+    constexpr int TILE = S_THREADS * EPV;
+    for (int tile = 0; tile < vocab; tile += TILE) {
+        const int base = tile + tid * EPV;
+        uint32_t keys[EPV];
+        if (vec && base + EPV <= vocab) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(rp + base);
+            const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) keys[j] = elem_key<T>(e[j], temp, has_t);
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPV; ++j)
+                keys[j] = (base + j < vocab) ? elem_key<T>(rp[base + j], temp, has_t) : 0u;
+        }
+        uint32_t tie_rank = 0;
+        if (track_ties) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) c += (base + j < vocab && keys[j] == kcut) ? 1u : 0u;
+            uint32_t tot;
+            tie_rank = carry_ties + block_excl_scan<uint32_t>(c, sh.wave_u32, &tot);
+            carry_ties += tot;
+        }
+        uint64_t w[EPV];
+        uint64_t msum = 0;
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) {
+            bool member = false;
+            if (base + j < vocab) {
+                if (keys[j] > kcut) member = true;
+                else if (keys[j] == kcut && keys[j] >= kstar) member = !track_ties || (tie_rank++ < r_cut);
+            }
+            w[j] = member ? weight_fix(keys[j] == kmax ? 0.0f : value_of(keys[j]) - vmax) : 0ull;
+            msum += w[j];
+        }
+        uint64_t tot;
+        const uint64_t excl = carry_mass + block_excl_scan<uint64_t>(msum, sh.wave_u64, &tot);
+        if (excl <= tau && tau < excl + msum) {
+            uint64_t cum = excl;
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) {
+                cum += w[j];
+                if (cum > tau) { sh.hit = base + j; break; }
+            }
+        }
+        carry_mass += tot;
+        if (carry_mass > tau) break;  // block-uniform: the hit lies in this tile
+    }
+    __syncthreads();
+    if (tid == 0) out[row] = sh.hit;
+}
+
+template <typename T>
+int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride, float temperature,
+           int32_t top_k, float top_p, const float *uniforms, int64_t *out_ids, void *workspace,
+           size_t workspace_bytes, void *hip_stream) {
+    if (batch < 0) return fail(KA_ERR_BAD_ARG, "sample: batch %lld < 0", (long long)batch);
+    if (batch == 0) return KA_OK;
+    if (logits == nullptr || uniforms == nullptr || out_ids == nullptr)
+        return fail(KA_ERR_BAD_ARG, "sample: null logits / uniforms / out_ids pointer");
+    if (vocab < 1) return fail(KA_ERR_BAD_ARG, "sample: vocab %lld < 1", (long long)vocab);
+    if (vocab >= (int64_t(1) << 22))
+        return fail(KA_ERR_UNSUPPORTED, "sample: vocab %lld >= 2^22 (integer masses would overflow)",
+                    (long long)vocab);
+    if (row_stride < vocab) return fail(KA_ERR_BAD_ARG, "sample: row_stride < vocab");
+    if (!(temperature > 0.0f)) return fail(KA_ERR_BAD_ARG, "sample: temperature %g must be > 0", temperature);
+    if (top_k < 0) return fail(KA_ERR_BAD_ARG, "sample: top_k %d < 0", top_k);
+    if (!(top_p > 0.0f && top_p <= 1.0f)) return fail(KA_ERR_BAD_ARG, "sample: top_p %g outside (0, 1]", top_p);
+    if (batch >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "sample: batch too large");
+    if (workspace_bytes < ka_sample_workspace_bytes(batch, vocab) || (workspace == nullptr && workspace_bytes > 0))
+        return fail(KA_ERR_WORKSPACE, "sample: workspace of %zu B, need %zu B", workspace_bytes,
+                    ka_sample_workspace_bytes(batch, vocab));
+    const bool aligned = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * T::kBytes) % 16 == 0);
+    hipLaunchKernelGGL((sample_rows<T>), dim3(unsigned(batch)), dim3(S_THREADS), 0,
+                       static_cast<hipStream_t>(hip_stream),
+                       static_cast<const typename T::raw_t *>(logits), int(vocab), row_stride, temperature,
+                       int(top_k), top_p, uniforms, out_ids, aligned ? 1 : 0);
+    return check_hip(hipGetLastError(), "sample launch");
+}
+
+}  // namespace
+}  // namespace ka
+
+// The kernels keep all their state in LDS and registers; the workspace argument is reserved.
+KA_EXPORT size_t ka_sample_workspace_bytes(int64_t batch, int64_t vocab) {
+    (void)batch;
+    (void)vocab;
+    return 0;
+}
+
+KA_EXPORT int ka_sample_topk_topp_bf16(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                                       float temperature, int32_t top_k, float top_p, const float *uniforms,
+                                       int64_t *out_ids, void *workspace, size_t workspace_bytes,
+                                       void *hip_stream) {
+    return ka::launch<ka::Bf16>(logits, batch, vocab, row_stride, temperature, top_k, top_p, uniforms, out_ids,
+                                workspace, workspace_bytes, hip_stream);
+}
+KA_EXPORT int ka_sample_topk_topp_f16(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                                      float temperature, int32_t top_k, float top_p, const float *uniforms,
+                                      int64_t *out_ids, void *workspace, size_t workspace_bytes,
+                                      void *hip_stream) {
+    return ka::launch<ka::F16>(logits, batch, vocab, row_stride, temperature, top_k, top_p, uniforms, out_ids,
+                               workspace, workspace_bytes, hip_stream);
+}
+KA_EXPORT int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                                      float temperature, int32_t top_k, float top_p, const float *uniforms,
+                                      int64_t *out_ids, void *workspace, size_t workspace_bytes,
+                                      void *hip_stream) {
+    return ka::launch<ka::F32>(logits, batch, vocab, row_stride, temperature, top_k, top_p, uniforms, out_ids,
+                               workspace, workspace_bytes, hip_stream);
+}

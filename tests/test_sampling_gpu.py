@@ -1,0 +1,151 @@
+"""Parity of the HIP sampling kernel (through the C ABI) with the CPU oracles.  Needs an MI355X.
+
+Token ids must be bit-exact against oracle/ka_oracle.c (the exactly specified definition) on
+every row, and against the torch restatement of the reference's native_sampling on every row
+whose threshold decisions are not within fp32 rounding noise of a tie (on the BASELINE
+configuration that is every row).
+"""
+import math
+
+import pytest
+import torch
+
+from benchmarks.workloads import cfg5_sampling
+from oracle import exact, sampling_ref
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+def run(sampler, logits, u, k, p, temp):
+    return sampler.sample(logits.cuda(), top_k=k, top_p=p, temperature=temp, uniforms=u.cuda()).cpu()
+
+
+def check_exact(sampler, logits, u, k, p, temp):
+    got = run(sampler, logits, u, k, p, temp)
+    want = exact.sample(logits, temp, k, p, u)
+    assert got.dtype == torch.int64 and got.shape == want.shape
+    bad = (got != want).nonzero().flatten().tolist()
+    assert not bad, f"rows {bad[:8]}: got {got[bad[:8]].tolist()} want {want[bad[:8]].tolist()}"
+    return got
+
+
+@pytest.mark.parametrize("batch", [64, 128, 256])
+def test_baseline_config_bit_exact(sampler, batch):
+    logits, u = cfg5_sampling(batch)
+    got = check_exact(sampler, logits, u, 50, 0.9, 0.7)
+    ref, margin = sampling_ref.sample(logits, 50, 0.9, 0.7, u)
+    assert margin.min().item() > 1e-6
+    assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k,p,temp", [(50, 0.9, 0.7), (50, None, 1.0), (None, 0.9, 1.0), (None, None, 1.0),
+                                      (None, None, 0.7), (1, None, 1.0), (1, 0.5, 1.3), (5000, 0.99, 0.5),
+                                      (50, 1e-6, 1.0), (2, 1.0, 1.0)])
+def test_modes_and_dtypes(sampler, dtype, k, p, temp):
+    g = torch.Generator().manual_seed(21)
+    logits = (torch.randn(48, 32000, generator=g) * 3).to(dtype)
+    u = torch.rand(48, generator=g)
+    got = check_exact(sampler, logits, u, k, p, temp)
+    ref, margin = sampling_ref.sample(logits, k, p, temp, u)
+    differ = got != ref
+    assert (margin[differ] < 1e-6).all() and differ.sum().item() <= 1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k,p,temp", [(5, 0.9, 0.7), (5, None, 1.0), (None, 0.8, 1.0), (17, 0.05, 1.0),
+                                      (200, 0.95, 0.5), (3, 1.0, 2.0)])
+def test_heavy_ties_and_degenerate_rows(sampler, dtype, k, p, temp):
+    g = torch.Generator().manual_seed(22)
+    logits = ((torch.randn(40, 3000, generator=g) * 12).round() / 4).to(dtype)
+    u = torch.rand(40, generator=g)
+    logits[0, :] = 1.5                       # all equal: every entry ties at the k-th value and at the cut
+    logits[1, :] = -math.inf                 # only -inf
+    logits[2, 7] = math.inf                  # +inf wins outright
+    logits[3, :2500] = -math.inf             # masked prefix
+    logits[4, :] = 0.0
+    logits[4, 100:200] = -0.0                # signed zeros are one value
+    logits[5, 5] = 30.0                      # one dominant entry: everything else has mass ~0
+    check_exact(sampler, logits, u, k, p, temp)
+
+
+def test_all_equal_llama_row_cut_inside_tie_group(sampler):
+    logits = torch.zeros(4, 128256, dtype=torch.bfloat16)
+    u = torch.tensor([0.0, 0.25, 0.5, 0.999])
+    got = check_exact(sampler, logits, u, 50, 0.3, 0.7)
+    kept = math.floor(float(torch.tensor(0.3, dtype=torch.float32)) * 128256) + 1
+    assert got.tolist() == [math.floor(float(x) * kept) for x in u]
+
+
+@pytest.mark.parametrize("vocab", [1, 2, 7, 8, 9, 63, 1000, 2047, 8193, 32003, 151936])
+def test_ragged_vocab(sampler, vocab):
+    g = torch.Generator().manual_seed(vocab)
+    logits = (torch.randn(6, vocab, generator=g) * 3).bfloat16()
+    u = torch.rand(6, generator=g)
+    check_exact(sampler, logits, u, 50, 0.9, 0.7)
+    check_exact(sampler, logits, u, None, 0.9, 1.0)
+
+
+def test_unaligned_and_strided_rows(sampler):
+    g = torch.Generator().manual_seed(23)
+    big = (torch.randn(12, 4104, generator=g) * 3).bfloat16()
+    u = torch.rand(12, generator=g)
+    for view in (big[:, 3:4004], big[:, 8:4009], big[:, :4096]):
+        got = sampler.sample(view.cuda(), top_k=20, top_p=0.9, temperature=0.7, uniforms=u.cuda()).cpu()
+        assert torch.equal(got, exact.sample(view.contiguous(), 0.7, 20, 0.9, u))
+
+
+def test_extreme_uniforms(sampler):
+    logits, _ = cfg5_sampling(8, vocab=32000)
+    for val in (0.0, 2.0 ** -149, 1 - 2.0 ** -24, 1.0, 7.0, -1.0, float("nan")):
+        check_exact(sampler, logits, torch.full((8,), val), 50, 0.9, 0.7)
+
+
+def test_every_bf16_value_through_the_temperature_step(sampler):
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = bits[torch.isfinite(bits.float())]
+    g = torch.Generator().manual_seed(24)
+    rows = torch.stack([finite[torch.randperm(finite.numel(), generator=g)] for _ in range(4)])
+    rows = torch.where(rows.float().abs() > 60, torch.zeros_like(rows), rows)   # keep exp() in range
+    u = torch.rand(4, generator=g)
+    for temp in (0.7, 1.3, 0.01):
+        check_exact(sampler, rows, u, 300, 0.95, temp)
+
+
+def test_bit_identical_across_runs_and_batch_splits(sampler):
+    logits, u = cfg5_sampling(256)
+    dl, du = logits.cuda(), u.cuda()
+    base = sampler.sample(dl, top_k=50, top_p=0.9, temperature=0.7, uniforms=du)
+    for _ in range(3):
+        assert torch.equal(base, sampler.sample(dl, top_k=50, top_p=0.9, temperature=0.7, uniforms=du))
+    for split in (1, 64, 100):
+        parts = [sampler.sample(dl[s:s + split], top_k=50, top_p=0.9, temperature=0.7, uniforms=du[s:s + split])
+                 for s in range(0, 256, split)][:6]
+        cat = torch.cat(parts)
+        assert torch.equal(base[:cat.numel()], cat)
+
+
+def test_reference_call_shapes_and_generated_uniforms(sampler):
+    logits = torch.randn(16, 128256, device="cuda")                      # fp32, as benchmark_sampling.py:58
+    ids = sampler.sample(logits, top_k=50, top_p=0.9)
+    assert ids.shape == (16,) and ids.dtype == torch.int64 and ids.device.type == "cuda"
+    assert ((ids >= 0) & (ids < 128256)).all()
+    g1 = torch.Generator(device="cuda").manual_seed(5)
+    g2 = torch.Generator(device="cuda").manual_seed(5)
+    assert torch.equal(sampler.sample(logits, top_k=50, generator=g1), sampler.sample(logits, top_k=50, generator=g2))
+    top1 = sampler.sample(logits, top_k=1)
+    assert torch.equal(top1, logits.argmax(dim=-1))
+    assert sampler.sample(logits[:0], top_k=5).shape == (0,)
+
+
+def test_invalid_arguments_raise(sampler):
+    logits = torch.zeros(2, 64, dtype=torch.bfloat16, device="cuda")
+    for kw in (dict(top_k=0), dict(top_k=-3), dict(top_p=0.0), dict(top_p=1.5), dict(temperature=0.0),
+               dict(temperature=-1.0)):
+        with pytest.raises(ValueError):
+            sampler.sample(logits, **kw)
+    with pytest.raises(RuntimeError):
+        sampler.sample(logits.cpu(), top_k=5)
+    with pytest.raises(ValueError):
+        sampler.sample(logits, uniforms=torch.zeros(3, device="cuda"))
