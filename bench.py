@@ -58,6 +58,36 @@ def cpu_baseline(logits, ids, sample_rows: int):
     }
 
 
+def sampling_latency(sampler, steps: int, warmup: int):
+    """Fused sampling on bf16 [B, 128256], T=0.7, top-k 50, top-p 0.9, uniforms from seed 1234."""
+    import torch
+    from benchmarks.workloads import cfg5_sampling
+
+    out = {"config": "bf16 [B,128256] ~ N(0,3^2), T=0.7, top_k=50, top_p=0.9, one fp32 uniform per row (seed 1234)"}
+    for batch in (64, 128, 256):
+        logits, u = cfg5_sampling(batch, device="cuda")
+        for _ in range(max(warmup, 3)):
+            sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = max(steps, 20)
+        t0 = time.perf_counter()
+        ev0.record()
+        for _ in range(n):
+            sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u)
+        ev1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / n
+        kernel_ms = ev0.elapsed_time(ev1) / n
+        out[f"ms_b{batch}"] = wall_ms
+        out[f"kernel_ms_b{batch}"] = kernel_ms
+        if batch == 256:
+            gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
+            out["roofline"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                               "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel": "sample_rows<Bf16>"}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,6 +106,10 @@ def main() -> int:
         return 2
 
     import torch
+    from rl_engine.utils.logger import logger
+
+    for handler in logger.handlers:  # stdout carries the JSON line only
+        handler.setStream(sys.stderr)
     from benchmarks.workloads import spike_logits
     from rl_engine.kernels import sampling as sampling_mod
     from rl_engine.kernels.sampling import SamplerBackend
@@ -146,6 +180,8 @@ def main() -> int:
                      "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
     }
     assert bool(torch.isfinite(out).all()), "non-finite logprob in the timed run"
+    del logits3, ids2
+    result["sampling"] = sampling_latency(sampler, args.steps, args.warmup)
     if args.cpu_sample_rows > 0:
         log("timing the CPU oracle on a sample of the same tensor")
         result["cpu_baseline"] = cpu_baseline(logits, ids, args.cpu_sample_rows)

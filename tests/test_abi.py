@@ -1,0 +1,74 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and rejects bad
+arguments with the documented status codes.  No kernel is launched here."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from rl_engine.kernels import _hip
+
+REPO = Path(__file__).resolve().parents[1]
+HEADER = REPO / "include" / "kernel_align_hip.h"
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(ka_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_binding_and_library_agree():
+    names = declared_symbols()
+    assert len(names) >= 13
+    assert sorted(_hip.SIGNATURES) == names, "ctypes binding and header list different entry points"
+    lib = _hip.load()
+    for name in names:
+        assert getattr(lib, name) is not None
+
+
+def test_version_and_status_strings():
+    lib = _hip.load()
+    assert b"gfx950" in lib.ka_version()
+    assert lib.ka_status_string(0) == b"KA_OK"
+    assert lib.ka_status_string(-1) == b"KA_ERR_BAD_ARG"
+    assert lib.ka_status_string(-3) == b"KA_ERR_WORKSPACE"
+    assert lib.ka_status_string(-99) == b"KA_ERR_UNKNOWN"
+
+
+def test_logprob_argument_checks():
+    lib = _hip.load()
+    p = ctypes.c_void_p(4096)
+    assert lib.ka_logprob_bf16(None, 0, 128, 128, None, None, None) == _hip.KA_OK          # empty batch
+    assert lib.ka_logprob_bf16(None, 4, 128, 128, p, p, None) == _hip.KA_ERR_BAD_ARG
+    assert b"null" in lib.ka_last_error()
+    assert lib.ka_logprob_bf16(p, -1, 128, 128, p, p, None) == _hip.KA_ERR_BAD_ARG
+    assert lib.ka_logprob_f32(p, 4, 0, 128, p, p, None) == _hip.KA_ERR_BAD_ARG
+    assert lib.ka_logprob_f16(p, 4, 128, 64, p, p, None) == _hip.KA_ERR_BAD_ARG              # stride < vocab
+    assert lib.ka_logprob_bf16(p, 4, 1 << 31, 1 << 31, p, p, None) == _hip.KA_ERR_UNSUPPORTED
+    with pytest.raises(ValueError, match="KA_ERR_BAD_ARG"):
+        _hip.check(lib.ka_logprob_bf16(p, 4, 128, 64, p, p, None), "ka_logprob_bf16")
+
+
+def test_sampling_argument_checks():
+    lib = _hip.load()
+    p = ctypes.c_void_p(4096)
+    call = lib.ka_sample_topk_topp_bf16
+    assert call(None, 0, 128, 128, 1.0, 0, 1.0, None, None, None, 0, None) == _hip.KA_OK
+    assert call(None, 2, 128, 128, 1.0, 0, 1.0, p, p, None, 0, None) == _hip.KA_ERR_BAD_ARG
+    assert call(p, 2, 128, 128, 0.0, 0, 1.0, p, p, None, 0, None) == _hip.KA_ERR_BAD_ARG    # temperature
+    assert call(p, 2, 128, 128, 1.0, -1, 1.0, p, p, None, 0, None) == _hip.KA_ERR_BAD_ARG   # top_k
+    assert call(p, 2, 128, 128, 1.0, 5, 0.0, p, p, None, 0, None) == _hip.KA_ERR_BAD_ARG    # top_p
+    assert call(p, 2, 128, 128, 1.0, 5, 1.5, p, p, None, 0, None) == _hip.KA_ERR_BAD_ARG
+    assert call(p, 2, 1 << 22, 1 << 22, 1.0, 5, 0.9, p, p, None, 0, None) == _hip.KA_ERR_UNSUPPORTED
+    assert lib.ka_sample_workspace_bytes(256, 128256) >= 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setenv(_hip.ENV_LIB, str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_hip, "_lib", None)
+    with pytest.raises(_hip.HipLibraryError, match="not found"):
+        _hip.load()
+    from rl_engine.kernels.sampling import SamplerBackend
+
+    with pytest.raises(_hip.HipLibraryError):
+        SamplerBackend()

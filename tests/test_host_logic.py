@@ -1,0 +1,87 @@
+"""Host side of the op API on a machine without a GPU: construction, validation, pool, side API."""
+import pytest
+import torch
+
+from rl_engine.executors.rollout import RolloutExecutor
+from rl_engine.kernels.pool import MAX_POOL_BYTES, PoolExhausted, WorkspacePool
+from rl_engine.kernels.registry import OpBackend, kernel_registry
+from rl_engine.kernels.sampling import SamplerBackend
+from rl_engine.platforms.device import device_ctx
+from rl_engine.utils.logger import logger
+
+
+def test_sampler_constructs_like_the_reference_module():
+    s = SamplerBackend()
+    assert isinstance(s, torch.nn.Module) and list(s.parameters()) == []
+    assert s.backend == "hip_native"
+    assert s.to("cpu") is s
+
+
+def test_no_cpu_path():
+    s = SamplerBackend()
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        s.compute_logp(torch.zeros(2, 3, 8, dtype=torch.bfloat16), torch.zeros(2, 3, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        s.sample(torch.zeros(2, 8), top_k=2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        s.fused_linear_logp(torch.zeros(2, 8, dtype=torch.bfloat16), torch.zeros(4, 8, dtype=torch.bfloat16),
+                            torch.zeros(2, dtype=torch.int64))
+
+
+def test_pool_is_fixed_size_and_never_grows():
+    pool = WorkspacePool(1 << 20)
+    assert pool.capacity == 1 << 20 and pool.allocated_bytes() == 0
+    with pytest.raises(ValueError):
+        WorkspacePool(MAX_POOL_BYTES + 1)
+    with pytest.raises(ValueError):
+        WorkspacePool(0)
+    pool._arenas[0] = torch.empty(pool.capacity, dtype=torch.uint8)   # stand-in arena on the CPU
+    dev = torch.device("cuda", 0)
+    a = pool.reserve(1000, dev)
+    b = pool.reserve(5000, dev)
+    assert a.numel() == 1000 and b.numel() == 5000
+    assert b.data_ptr() - a.data_ptr() == 1024 and b.data_ptr() % 256 == a.data_ptr() % 256
+    with pytest.raises(PoolExhausted):
+        pool.reserve(1 << 20, dev)
+    pool.reset()
+    assert pool.reserve(1 << 20, dev).numel() == 1 << 20
+
+
+def test_device_context_and_logger():
+    assert device_ctx.get_preferred_dtype() == torch.bfloat16
+    assert device_ctx.device_type in ("rocm", "cpu")
+    assert device_ctx.is_rocm == torch.cuda.is_available()
+    seen = []
+    import logging
+
+    class Grab(logging.Handler):
+        def emit(self, record):
+            seen.append(record.getMessage())
+
+    h = Grab()
+    logger.addHandler(h)
+    try:
+        for _ in range(3):
+            logger.info_once("only once %s", "x")
+        logger.warn_once("warn once")
+        logger.warn_once("warn once")
+        logger.info_on_rank("rank zero")
+        logger.info_on_rank("rank one", 1)
+    finally:
+        logger.removeHandler(h)
+    assert seen == ["only once x", "warn once", "rank zero"]
+
+
+def test_registry_and_executor():
+    assert kernel_registry.dispatch("fused_logp") == "HIP_LOGPROB"
+    assert kernel_registry.dispatch("sampling") == "HIP_SAMPLING"
+    assert kernel_registry.dispatch("fused_lm_head_logp") == "HIP_FUSED_LMHEAD_LOGPROB"
+    assert kernel_registry.get_op_path(OpBackend.HIP_LOGPROB).endswith("SamplerBackend.compute_logp")
+    with pytest.raises(ValueError):
+        kernel_registry.dispatch("attention")
+    with pytest.raises(ValueError, match="Supported backends"):
+        OpBackend["FLASHINFER"]
+    fn = kernel_registry.resolve("fused_logp")
+    assert fn.__name__ == "compute_logp"
+    out = RolloutExecutor({"top_k": 50}).execute_rollout()
+    assert out == {"status": "success", "kernels": ["HIP_LOGPROB", "HIP_SAMPLING"]}
