@@ -1,9 +1,330 @@
-// Fused lm_head -> logprob (placeholder entry points while the kernel is being written).
+// Fused lm_head -> logprob: out[n] = h_n . W[id_n] - logsumexp_v(h_n . W[v]),
+// without materialising the [n_rows, vocab] logits.
+//
+// Tiling (gfx950, wave64, v_mfma_f32_32x32x16_bf16):
+//   * a workgroup of 4 wavefronts owns 256 tokens and walks a range of 256-row
+//     vocabulary tiles; per tile it runs a K loop over the hidden dimension in
+//     slabs of 32, staging the W slab [256 x 32] and the hidden slab [256 x 32]
+//     through double-buffered, XOR-swizzled LDS (64 KB);
+//   * the MFMA "A" operand is W (rows of the result = vocabulary entries) and
+//     "B" is hidden (columns = tokens), so every lane's 64 accumulators of one
+//     32-column block belong to ONE token: the online max / sum-of-exp update
+//     after each vocabulary tile is register-local, with no cross-lane traffic;
+//   * each wavefront computes 128 vocab x 128 tokens = 4 x 4 MFMA blocks
+//     (256 fp32 accumulators per lane);
+//   * the vocabulary is cut into fixed splits of LM_TILES_PER_SPLIT tiles (a
+//     function of the vocabulary only, so results do not depend on the number of
+//     rows); every (token block, split) writes one (max, sum, target logit)
+//     partial per token and a second kernel folds the partials in split order.
+// Logits stay in fp32 (the accumulators are not rounded to bf16).
 #include "ka_common.h"
 
-KA_EXPORT size_t ka_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab) { return 256; }
+namespace ka {
+namespace {
 
-KA_EXPORT int ka_lmhead_logprob_bf16(const void *, const void *, const int64_t *, float *, int64_t, int64_t,
-                                     int64_t, void *, size_t, void *) {
-    return ka::fail(KA_ERR_UNSUPPORTED, "ka_lmhead_logprob_bf16: not implemented");
+constexpr int LM_BM = 256;      // vocabulary rows per tile
+constexpr int LM_BN = 256;      // tokens per workgroup
+constexpr int LM_BK = 32;       // hidden slab
+constexpr int LM_THREADS = 256;
+constexpr int LM_TILES_PER_SPLIT = 63;
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr double kLn2 = 0.693147180559945309417232;
+constexpr float kFloor = -1.0e30f;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct Partial {
+    float m;   // max logit seen (>= kFloor)
+    float s;   // sum of exp(logit - m)
+    float xt;  // target logit if this split holds it, else -inf
+    float pad;
+};
+
+// LDS slab: 256 rows x 32 bf16 (64 B per row = four 16-byte chunks), chunk index
+// XOR-swizzled with the row so that eight consecutive rows land in eight different
+// 16-byte columns of a 128-byte bank line.
+__device__ __forceinline__ int slab_offset(int row, int chunk) {
+    return row * 32 + ((chunk ^ ((row >> 1) & 3)) << 3);  // in bf16 elements
+}
+
+__global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
+    const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
+    Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_splits, int n_token_blocks,
+    int n_vtiles) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2][2][LM_BM * LM_BK];  // [buffer][A=W / B=hidden]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave >> 1;  // which 128 vocabulary rows of the tile
+    const int wave_n = wave & 1;   // which 128 tokens of the block
+    const int l32 = lane & 31;
+    const int lhalf = lane >> 5;
+
+    // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
+    // (token block, split) pairs so that its L2 sees few distinct W and hidden tiles.
+    const int total = n_token_blocks * n_splits;
+    int logical = blockIdx.x;
+    if (total % 8 == 0) logical = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const int tb = logical / n_splits;
+    const int sp = logical % n_splits;
+    const int tok0 = tb * LM_BN;
+    const int vt_begin = sp * LM_TILES_PER_SPLIT;
+    const int vt_end = min(n_vtiles, vt_begin + LM_TILES_PER_SPLIT);
+    const int nk = hdim / LM_BK;
+
+    // This lane's four tokens (one per 32-column block of the wave tile) and their targets.
+    float m_run[4], ml2_run[4], s_run[4], xt[4];  // ml2_run = m_run * log2(e), kept so that it is never recomputed
+    int target[4];
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+        m_run[tn] = kFloor;
+        ml2_run[tn] = kFloor * kLog2e;
+        s_run[tn] = 0.0f;
+        xt[tn] = -__builtin_inff();
+        const int n = tok0 + wave_n * 128 + tn * 32 + l32;
+        int64_t id = -1;
+        if (n < n_rows) id = ids[n];
+        target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
+    }
+
+    // Global -> register staging: thread t moves chunk (t % 4) of rows t/4 + 64*i, i = 0..3.
+    // (Plain named registers: arrays captured by a lambda end up in scratch / LDS.)
+    const int ld_chunk = tid & 3;
+    const int ld_row = tid >> 2;
+    const int lds_st = slab_offset(ld_row, ld_chunk);  // rows +64*i keep the same swizzle (64 % 8 == 0)
+    const uint16_t *const h0 = hidden + size_t(min(tok0 + ld_row, n_rows - 1)) * hdim + ld_chunk * 8;
+    const uint16_t *const h1 = hidden + size_t(min(tok0 + ld_row + 64, n_rows - 1)) * hdim + ld_chunk * 8;
+    const uint16_t *const h2 = hidden + size_t(min(tok0 + ld_row + 128, n_rows - 1)) * hdim + ld_chunk * 8;
+    const uint16_t *const h3 = hidden + size_t(min(tok0 + ld_row + 192, n_rows - 1)) * hdim + ld_chunk * 8;
+    const uint16_t *const wbase = weight + ld_chunk * 8;
+    uint4 sa0, sa1, sa2, sa3, sb0, sb1, sb2, sb3;
+
+#define LM_LOAD_GLOBAL(vt_, kt_)                                                                       \
+    do {                                                                                               \
+        const int k_ = (kt_) * LM_BK;                                                                  \
+        const int v_ = (vt_) * LM_BM + ld_row;                                                         \
+        sa0 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_, vocab - 1)) * hdim + k_);        \
+        sa1 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_ + 64, vocab - 1)) * hdim + k_);   \
+        sa2 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_ + 128, vocab - 1)) * hdim + k_);  \
+        sa3 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_ + 192, vocab - 1)) * hdim + k_);  \
+        sb0 = *reinterpret_cast<const uint4 *>(h0 + k_);                                               \
+        sb1 = *reinterpret_cast<const uint4 *>(h1 + k_);                                               \
+        sb2 = *reinterpret_cast<const uint4 *>(h2 + k_);                                               \
+        sb3 = *reinterpret_cast<const uint4 *>(h3 + k_);                                               \
+    } while (0)
+#define LM_STORE_LDS(buf_)                                                                             \
+    do {                                                                                               \
+        uint16_t *pa_ = &lds[buf_][0][lds_st];                                                         \
+        uint16_t *pb_ = &lds[buf_][1][lds_st];                                                         \
+        *reinterpret_cast<uint4 *>(pa_) = sa0;                                                         \
+        *reinterpret_cast<uint4 *>(pa_ + 64 * LM_BK) = sa1;                                            \
+        *reinterpret_cast<uint4 *>(pa_ + 128 * LM_BK) = sa2;                                           \
+        *reinterpret_cast<uint4 *>(pa_ + 192 * LM_BK) = sa3;                                           \
+        *reinterpret_cast<uint4 *>(pb_) = sb0;                                                         \
+        *reinterpret_cast<uint4 *>(pb_ + 64 * LM_BK) = sb1;                                            \
+        *reinterpret_cast<uint4 *>(pb_ + 128 * LM_BK) = sb2;                                           \
+        *reinterpret_cast<uint4 *>(pb_ + 192 * LM_BK) = sb3;                                           \
+    } while (0)
+
+    LM_LOAD_GLOBAL(vt_begin, 0);
+    LM_STORE_LDS(0);
+    __syncthreads();
+
+    int buf = 0;
+    for (int vt = vt_begin; vt < vt_end; ++vt) {
+        f32x16 acc[4][4];
+#pragma unroll
+        for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
+
+        for (int kt = 0; kt < nk; ++kt) {
+            // prefetch the next slab (of this tile, or the first slab of the next tile)
+            const bool last_k = kt + 1 == nk;
+            const bool has_next = !last_k || vt + 1 < vt_end;
+            if (has_next) LM_LOAD_GLOBAL(last_k ? vt + 1 : vt, last_k ? 0 : kt + 1);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                bf16x8 a[4], b[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    a[t] = *reinterpret_cast<const bf16x8 *>(&lds[buf][0][slab_offset(wave_m * 128 + t * 32 + l32, kk * 2 + lhalf)]);
+                    b[t] = *reinterpret_cast<const bf16x8 *>(&lds[buf][1][slab_offset(wave_n * 128 + t * 32 + l32, kk * 2 + lhalf)]);
+                }
+#pragma unroll
+                for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < 4; ++tn)
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[tm], b[tn], acc[tm][tn], 0, 0, 0);
+            }
+            if (has_next) LM_STORE_LDS(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+
+        // ---- the logits of this vocabulary tile are complete: fold them into the running state ----
+        // Vocabulary row of acc[tm][tn][r]: vrow0 + tm*32 + (r/4)*8 + r%4.
+        const int vrow0 = vt * LM_BM + wave_m * 128 + lhalf * 4;
+        const int limit = vocab - vrow0;  // rows at offset >= limit lie past the vocabulary (last tile only)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            // keep the four token blocks apart: only 64 accumulators are live in VGPRs at a time
+            __builtin_amdgcn_sched_barrier(0);
+            const int d = target[tn] - (vt * LM_BM + wave_m * 128);
+            const bool mine = d >= 0 && d < 128 && ((d >> 2) & 1) == lhalf;
+            const int want = mine ? (((d >> 5) << 4) | ((d & 31) >> 3 << 2) | (d & 3)) : -1;  // tm*16 + r
+            float mn = m_run[tn];
+#pragma unroll
+            for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
+                    mn = fmaxf(mn, x);
+                    if (want == tm * 16 + r) xt[tn] = x;
+                }
+            const float ml2n = mn * kLog2e;
+            float part[4];
+#pragma unroll
+            for (int tm = 0; tm < 4; ++tm) {
+                float e[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
+                    e[r] = fast_exp2(fmaf(x, kLog2e, -ml2n));
+                }
+#pragma unroll
+                for (int step = 1; step < 16; step <<= 1)
+#pragma unroll
+                    for (int r = 0; r + step < 16; r += 2 * step) e[r] += e[r + step];
+                part[tm] = e[0];
+            }
+            // difference of the two stored products: recomputing m_run * log2e here could be fused into an
+            // FMA against ml2n and return the rounding residue of a 1e30-sized product instead of 0
+            const float rescale = fast_exp2(ml2_run[tn] - ml2n);
+            s_run[tn] = fmaf(s_run[tn], rescale, (part[0] + part[1]) + (part[2] + part[3]));
+            m_run[tn] = mn;
+            ml2_run[tn] = ml2n;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- fold the two lane halves (rows 4..7 of each 8-row group live in lanes 32..63) ----
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+        const float om = __shfl_xor(m_run[tn], 32, kWave);
+        const float os = __shfl_xor(s_run[tn], 32, kWave);
+        const float ox = __shfl_xor(xt[tn], 32, kWave);
+        const float mm = fmaxf(m_run[tn], om);
+        const float lo_s = lhalf == 0 ? s_run[tn] : os, lo_m = lhalf == 0 ? m_run[tn] : om;
+        const float hi_s = lhalf == 0 ? os : s_run[tn], hi_m = lhalf == 0 ? om : m_run[tn];
+        s_run[tn] = lo_s * fast_exp2((lo_m - mm) * kLog2e) + hi_s * fast_exp2((hi_m - mm) * kLog2e);
+        m_run[tn] = mm;
+        xt[tn] = fmaxf(xt[tn], ox);
+    }
+    // ---- fold the two vocabulary halves of the tile through LDS (upper half -> lower half) ----
+    float *xch = reinterpret_cast<float *>(&lds[0][0][0]);  // [wave_n][tn][32][3]
+    __syncthreads();
+    if (wave_m == 1 && lhalf == 0) {
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 3;
+            p[0] = m_run[tn];
+            p[1] = s_run[tn];
+            p[2] = xt[tn];
+        }
+    }
+    __syncthreads();
+    if (wave_m == 0 && lhalf == 0) {
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            const float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 3;
+            const float om = p[0], os = p[1], ox = p[2];
+            const float mm = fmaxf(m_run[tn], om);
+            const float s = s_run[tn] * fast_exp2((m_run[tn] - mm) * kLog2e) + os * fast_exp2((om - mm) * kLog2e);
+            const int n = tok0 + wave_n * 128 + tn * 32 + l32;
+            if (n < n_rows) {
+                Partial out;
+                out.m = mm;
+                out.s = s;
+                out.xt = fmaxf(xt[tn], ox);
+                out.pad = 0.0f;
+                partials[size_t(sp) * n_rows + n] = out;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict__ partials,
+                                                      const int64_t *__restrict__ ids, float *__restrict__ out,
+                                                      int n_rows, int vocab, int n_splits) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= n_rows) return;
+    float mm = kFloor;
+    for (int sp = 0; sp < n_splits; ++sp) mm = fmaxf(mm, partials[size_t(sp) * n_rows + n].m);
+    float s = 0.0f, x = -__builtin_inff();
+    for (int sp = 0; sp < n_splits; ++sp) {  // fixed split order
+        const Partial p = partials[size_t(sp) * n_rows + n];
+        s += p.s * fast_exp2((p.m - mm) * kLog2e);
+        x = fmaxf(x, p.xt);
+    }
+    const int64_t id = ids[n];
+    if (id < 0 || id >= vocab) {
+        out[n] = __builtin_nanf("");
+        return;
+    }
+    const double lse = double(mm) + log2(double(s)) * kLn2;
+    out[n] = float(double(x) - lse);
+}
+
+inline int splits_for(int64_t vocab) {
+    const int64_t n_vtiles = (vocab + LM_BM - 1) / LM_BM;
+    return int((n_vtiles + LM_TILES_PER_SPLIT - 1) / LM_TILES_PER_SPLIT);
+}
+
+}  // namespace
+}  // namespace ka
+
+KA_EXPORT size_t ka_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab) {
+    (void)hidden_dim;
+    if (n_rows <= 0 || vocab <= 0) return 0;
+    return size_t(ka::splits_for(vocab)) * size_t(n_rows) * sizeof(ka::Partial);
+}
+
+KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                     int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
+                                     size_t workspace_bytes, void *hip_stream) {
+    using namespace ka;
+    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead: n_rows %lld < 0", (long long)n_rows);
+    if (n_rows == 0) return KA_OK;
+    if (hidden == nullptr || weight == nullptr || ids == nullptr || out == nullptr)
+        return fail(KA_ERR_BAD_ARG, "lmhead: null hidden / weight / ids / out pointer");
+    if (hidden_dim < 8 || vocab < 1) return fail(KA_ERR_BAD_ARG, "lmhead: hidden_dim %lld, vocab %lld", (long long)hidden_dim, (long long)vocab);
+    if (hidden_dim % LM_BK != 0)
+        return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden_dim %lld is not a multiple of %d", (long long)hidden_dim, LM_BK);
+    if (reinterpret_cast<uintptr_t>(hidden) % 16 != 0 || reinterpret_cast<uintptr_t>(weight) % 16 != 0)
+        return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden and weight must be 16-byte aligned");
+    if (n_rows >= (int64_t(1) << 31) || vocab >= (int64_t(1) << 31) || hidden_dim >= (int64_t(1) << 31))
+        return fail(KA_ERR_UNSUPPORTED, "lmhead: a dimension does not fit 31 bits");
+    const size_t need = ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab);
+    if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return fail(KA_ERR_WORKSPACE, "lmhead: workspace of %zu B (16-byte aligned) needed, got %zu B", need, workspace_bytes);
+    const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
+    const int n_splits = splits_for(vocab);
+    const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
+    const int64_t grid = int64_t(n_token_blocks) * n_splits;
+    if (grid >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "lmhead: grid too large");
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    Partial *partials = static_cast<Partial *>(workspace);
+    hipLaunchKernelGGL(lmhead_partials, dim3(unsigned(grid)), dim3(LM_THREADS), 0, stream,
+                       static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
+                       int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles);
+    int rc = check_hip(hipGetLastError(), "lmhead partials launch");
+    if (rc != KA_OK) return rc;
+    hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids, out,
+                       int(n_rows), int(vocab), n_splits);
+    return check_hip(hipGetLastError(), "lmhead combine launch");
 }

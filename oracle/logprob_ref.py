@@ -75,3 +75,21 @@ def logprob_bruteforce(row, target: int) -> float:
     m = max(row)
     total = math.fsum(math.exp(v - m) for v in row if v != -math.inf)
     return row[target] - (m + math.log(total))
+
+
+def lmhead_logprob_ref(hidden: torch.Tensor, weight: torch.Tensor, token_ids: torch.Tensor,
+                       dtype=torch.float32, chunk_rows: int = 256) -> torch.Tensor:
+    """Oracle of the fused lm_head -> logprob operator: logprob of `hidden @ weight.T` kept in `dtype`
+    (fp32 or fp64; the bf16 inputs are exact in both), i.e. compute_logp(lm_head(hidden)) of
+    rl_engine/kernels/sampling.py:92-112 with an unrounded linear layer."""
+    hdim = hidden.shape[-1]
+    rows = hidden.reshape(-1, hdim).cpu()
+    ids = token_ids.reshape(-1).to(torch.int64).cpu()
+    w = weight.cpu().to(dtype)
+    out = torch.empty(rows.shape[0], dtype=dtype)
+    for s in range(0, rows.shape[0], chunk_rows):
+        logits = torch.nn.functional.linear(rows[s:s + chunk_rows].to(dtype), w)
+        m = logits.max(dim=-1, keepdim=True).values
+        lse = m.squeeze(-1) + torch.log(torch.exp(logits - m).sum(dim=-1))
+        out[s:s + chunk_rows] = logits.gather(-1, ids[s:s + chunk_rows].unsqueeze(-1)).squeeze(-1) - lse
+    return out.view(tuple(hidden.shape[:-1]))
