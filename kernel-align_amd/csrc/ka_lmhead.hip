@@ -4,8 +4,9 @@
 // Tiling (gfx950, wave64, v_mfma_f32_32x32x16_bf16):
 //   * a workgroup of 4 wavefronts owns 256 tokens and walks a range of 256-row
 //     vocabulary tiles; per tile it runs a K loop over the hidden dimension in
-//     slabs of 32, staging the W slab [256 x 32] and the hidden slab [256 x 32]
-//     through double-buffered, XOR-swizzled LDS (64 KB);
+//     slabs of 64; the W slab [256 x 64] and the hidden slab [256 x 64] go from
+//     global memory straight into XOR-swizzled LDS (global_load_lds_dwordx4, no
+//     register staging), two stages of 64 KB, one barrier per slab;
 //   * the MFMA "A" operand is W (rows of the result = vocabulary entries) and
 //     "B" is hidden (columns = tokens), so every lane's 64 accumulators of one
 //     32-column block belong to ONE token: the online max / sum-of-exp update
@@ -24,7 +25,9 @@ namespace {
 
 constexpr int LM_BM = 256;      // vocabulary rows per tile
 constexpr int LM_BN = 256;      // tokens per workgroup
-constexpr int LM_BK = 32;       // hidden slab
+constexpr int LM_BK = 64;       // hidden slab
+constexpr int LM_STAGE_ELEMS = (LM_BM + LM_BN) * LM_BK;  // bf16 elements per LDS stage (64 KB)
+constexpr int LM_LDS_BYTES = 2 * LM_STAGE_ELEMS * 2;
 constexpr int LM_THREADS = 256;
 constexpr int LM_TILES_PER_SPLIT = 63;
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -41,18 +44,24 @@ struct Partial {
     float pad;
 };
 
-// LDS slab: 256 rows x 32 bf16 (64 B per row = four 16-byte chunks), chunk index
-// XOR-swizzled with the row so that eight consecutive rows land in eight different
-// 16-byte columns of a 128-byte bank line.
+// LDS slab: 256 rows x 64 bf16 (128 B per row = eight 16-byte chunks).  A fragment read
+// (ds_read_b128) has lane l fetch row l % 32 at logical chunk 2*kk + l / 32.  The chunk index is
+// XOR-swizzled with swz(row) = ((row & 3) << 1) | ((row >> 2) & 1): eight consecutive rows get eight
+// different values, and four consecutive rows get four different values in the bits above bit 0, so
+// lanes l..l+3 together with their partners l+32..l+35 (same rows, neighbouring chunk) also touch
+// eight different 16-byte columns.
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 __device__ __forceinline__ int slab_offset(int row, int chunk) {
-    return row * 32 + ((chunk ^ ((row >> 1) & 3)) << 3);  // in bf16 elements
+    return row * LM_BK + ((chunk ^ swz(row)) << 3);  // in bf16 elements
 }
+
+typedef __attribute__((address_space(3))) void lds_void;
 
 __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
     Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_splits, int n_token_blocks,
     int n_vtiles) {
-    __shared__ __attribute__((aligned(16))) uint16_t lds[2][2][LM_BM * LM_BK];  // [buffer][A=W / B=hidden]
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [stage][A = W slab | B = hidden slab]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -89,50 +98,37 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
     }
 
-    // Global -> register staging: thread t moves chunk (t % 4) of rows t/4 + 64*i, i = 0..3.
-    // (Plain named registers: arrays captured by a lambda end up in scratch / LDS.)
-    const int ld_chunk = tid & 3;
-    const int ld_row = tid >> 2;
-    const int lds_st = slab_offset(ld_row, ld_chunk);  // rows +64*i keep the same swizzle (64 % 8 == 0)
-    const uint16_t *const h0 = hidden + size_t(min(tok0 + ld_row, n_rows - 1)) * hdim + ld_chunk * 8;
-    const uint16_t *const h1 = hidden + size_t(min(tok0 + ld_row + 64, n_rows - 1)) * hdim + ld_chunk * 8;
-    const uint16_t *const h2 = hidden + size_t(min(tok0 + ld_row + 128, n_rows - 1)) * hdim + ld_chunk * 8;
-    const uint16_t *const h3 = hidden + size_t(min(tok0 + ld_row + 192, n_rows - 1)) * hdim + ld_chunk * 8;
-    const uint16_t *const wbase = weight + ld_chunk * 8;
-    uint4 sa0, sa1, sa2, sa3, sb0, sb1, sb2, sb3;
+    // Global -> LDS copies.  One global_load_lds_dwordx4 moves 16 B per lane to LDS base + 16 * lane,
+    // i.e. one wavefront fills eight consecutive 128-byte rows; instruction j of wavefront w covers rows
+    // (4j + w) * 8 .. + 7.  Lane l therefore fetches row (4j + w) * 8 + l / 8 and, because the slab is
+    // swizzled, the logical chunk (l % 8) ^ swz(l / 8).  Row offsets are 32-bit byte offsets from a
+    // wavefront-uniform base (the host checks that both matrices are smaller than 4 GiB).
+    const int cp_row = wave * 8 + (lane >> 3);                 // + 32 * j
+    const int cp_chunk = (lane & 7) ^ swz(lane >> 3);
+    uint32_t hoff[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        hoff[j] = uint32_t(min(tok0 + cp_row + 32 * j, n_rows - 1)) * uint32_t(hdim) * 2u + cp_chunk * 16u;
+    const int wave_lds = __builtin_amdgcn_readfirstlane(wave) * 512;  // bf16 elements: 8 rows of 64
+    const char *const wbytes = reinterpret_cast<const char *>(weight);
+    const char *const hbytes = reinterpret_cast<const char *>(hidden);
 
-#define LM_LOAD_GLOBAL(vt_, kt_)                                                                       \
-    do {                                                                                               \
-        const int k_ = (kt_) * LM_BK;                                                                  \
-        const int v_ = (vt_) * LM_BM + ld_row;                                                         \
-        sa0 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_, vocab - 1)) * hdim + k_);        \
-        sa1 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_ + 64, vocab - 1)) * hdim + k_);   \
-        sa2 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_ + 128, vocab - 1)) * hdim + k_);  \
-        sa3 = *reinterpret_cast<const uint4 *>(wbase + size_t(min(v_ + 192, vocab - 1)) * hdim + k_);  \
-        sb0 = *reinterpret_cast<const uint4 *>(h0 + k_);                                               \
-        sb1 = *reinterpret_cast<const uint4 *>(h1 + k_);                                               \
-        sb2 = *reinterpret_cast<const uint4 *>(h2 + k_);                                               \
-        sb3 = *reinterpret_cast<const uint4 *>(h3 + k_);                                               \
-    } while (0)
-#define LM_STORE_LDS(buf_)                                                                             \
-    do {                                                                                               \
-        uint16_t *pa_ = &lds[buf_][0][lds_st];                                                         \
-        uint16_t *pb_ = &lds[buf_][1][lds_st];                                                         \
-        *reinterpret_cast<uint4 *>(pa_) = sa0;                                                         \
-        *reinterpret_cast<uint4 *>(pa_ + 64 * LM_BK) = sa1;                                            \
-        *reinterpret_cast<uint4 *>(pa_ + 128 * LM_BK) = sa2;                                           \
-        *reinterpret_cast<uint4 *>(pa_ + 192 * LM_BK) = sa3;                                           \
-        *reinterpret_cast<uint4 *>(pb_) = sb0;                                                         \
-        *reinterpret_cast<uint4 *>(pb_ + 64 * LM_BK) = sb1;                                            \
-        *reinterpret_cast<uint4 *>(pb_ + 128 * LM_BK) = sb2;                                           \
-        *reinterpret_cast<uint4 *>(pb_ + 192 * LM_BK) = sb3;                                           \
+    // Requests slab (vt_, kt_) into LDS stage stage_.
+#define LM_ISSUE_LOADS(vt_, kt_, stage_)                                                                     \
+    do {                                                                                                     \
+        const size_t kb_ = size_t(kt_) * (LM_BK * 2);                                                        \
+        uint16_t *sa_ = lds + (stage_) * LM_STAGE_ELEMS + wave_lds;                                           \
+        uint16_t *sb_ = sa_ + LM_BM * LM_BK;                                                                 \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                                      \
+            const uint32_t woff_ = uint32_t(min((vt_) * LM_BM + cp_row + 32 * j, vocab - 1)) * uint32_t(hdim) * 2u + cp_chunk * 16u; \
+            __builtin_amdgcn_global_load_lds(wbytes + kb_ + woff_, (lds_void *)(sa_ + j * 2048), 16, 0, 0);  \
+            __builtin_amdgcn_global_load_lds(hbytes + kb_ + hoff[j], (lds_void *)(sb_ + j * 2048), 16, 0, 0); \
+        }                                                                                                    \
     } while (0)
 
-    LM_LOAD_GLOBAL(vt_begin, 0);
-    LM_STORE_LDS(0);
-    __syncthreads();
+    LM_ISSUE_LOADS(vt_begin, 0, 0);
 
-    int buf = 0;
+    int stage = 0;
     for (int vt = vt_begin; vt < vt_end; ++vt) {
         f32x16 acc[4][4];
 #pragma unroll
@@ -143,27 +139,57 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                 for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
         for (int kt = 0; kt < nk; ++kt) {
-            // prefetch the next slab (of this tile, or the first slab of the next tile)
+            // Slab (vt, kt) was requested one iteration ago.  Wait for this lane's copies, then meet the
+            // other wavefronts: after the barrier the whole slab is in LDS and nobody reads the other stage.
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's global->LDS copies have landed
+            __syncthreads();
+            // Request the next slab (of this tile, or the first of the next tile).  The very last iteration
+            // re-requests its own slab into the idle stage, so that this block has no branch and the copies
+            // can be interleaved with the MFMAs below.
             const bool last_k = kt + 1 == nk;
-            const bool has_next = !last_k || vt + 1 < vt_end;
-            if (has_next) LM_LOAD_GLOBAL(last_k ? vt + 1 : vt, last_k ? 0 : kt + 1);
+            const bool more = !last_k || vt + 1 < vt_end;
+            const int vt_n = more ? (last_k ? vt + 1 : vt) : vt;
+            const int kt_n = more ? (last_k ? 0 : kt + 1) : kt;
+            LM_ISSUE_LOADS(vt_n, kt_n, stage ^ 1);
+
+            const uint16_t *sa = lds + stage * LM_STAGE_ELEMS;
+            const uint16_t *sb = sa + LM_BM * LM_BK;
+            bf16x8 fa[2][4], fb[2][4];
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                bf16x8 a[4], b[4];
+            for (int t = 0; t < 4; ++t) {
+                fa[0][t] = *reinterpret_cast<const bf16x8 *>(sa + slab_offset(wave_m * 128 + t * 32 + l32, lhalf));
+                fb[0][t] = *reinterpret_cast<const bf16x8 *>(sb + slab_offset(wave_n * 128 + t * 32 + l32, lhalf));
+            }
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    a[t] = *reinterpret_cast<const bf16x8 *>(&lds[buf][0][slab_offset(wave_m * 128 + t * 32 + l32, kk * 2 + lhalf)]);
-                    b[t] = *reinterpret_cast<const bf16x8 *>(&lds[buf][1][slab_offset(wave_n * 128 + t * 32 + l32, kk * 2 + lhalf)]);
+            for (int kk = 0; kk < 4; ++kk) {
+                if (kk < 3) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        fa[(kk + 1) & 1][t] = *reinterpret_cast<const bf16x8 *>(
+                            sa + slab_offset(wave_m * 128 + t * 32 + l32, (kk + 1) * 2 + lhalf));
+                        fb[(kk + 1) & 1][t] = *reinterpret_cast<const bf16x8 *>(
+                            sb + slab_offset(wave_n * 128 + t * 32 + l32, (kk + 1) * 2 + lhalf));
+                    }
                 }
 #pragma unroll
                 for (int tm = 0; tm < 4; ++tm)
 #pragma unroll
                     for (int tn = 0; tn < 4; ++tn)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[tm], b[tn], acc[tm][tn], 0, 0, 0);
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][tm], fb[kk & 1][tn],
+                                                                              acc[tm][tn], 0, 0, 0);
             }
-            if (has_next) LM_STORE_LDS(buf ^ 1);
-            __syncthreads();
-            buf ^= 1;
+            // Instruction order for this block: the 8 fragment reads of the first k-step, then every pair of
+            // MFMAs is followed by one fragment read of the next k-step and (for the first 16 pairs) one
+            // global->LDS copy, so that neither LDS latency nor copy issue leaves the matrix pipe idle.
+            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+            for (int i = 0; i < 24; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (i < 16) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+            stage ^= 1;
         }
 
         // ---- the logits of this vocabulary tile are complete: fold them into the running state ----
@@ -226,7 +252,8 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         xt[tn] = fmaxf(xt[tn], ox);
     }
     // ---- fold the two vocabulary halves of the tile through LDS (upper half -> lower half) ----
-    float *xch = reinterpret_cast<float *>(&lds[0][0][0]);  // [wave_n][tn][32][3]
+    float *xch = reinterpret_cast<float *>(lds);  // [wave_n][tn][32][3]
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the last (redundant) slab request may still be writing LDS
     __syncthreads();
     if (wave_m == 1 && lhalf == 0) {
 #pragma unroll
@@ -309,6 +336,8 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
         return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden and weight must be 16-byte aligned");
     if (n_rows >= (int64_t(1) << 31) || vocab >= (int64_t(1) << 31) || hidden_dim >= (int64_t(1) << 31))
         return fail(KA_ERR_UNSUPPORTED, "lmhead: a dimension does not fit 31 bits");
+    if (n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32))
+        return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden or weight matrix of 4 GiB or more (32-bit row offsets)");
     const size_t need = ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab);
     if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
         return fail(KA_ERR_WORKSPACE, "lmhead: workspace of %zu B (16-byte aligned) needed, got %zu B", need, workspace_bytes);
@@ -319,7 +348,10 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     if (grid >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "lmhead: grid too large");
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     Partial *partials = static_cast<Partial *>(workspace);
-    hipLaunchKernelGGL(lmhead_partials, dim3(unsigned(grid)), dim3(LM_THREADS), 0, stream,
+    static const hipError_t attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials),
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
+    if (attr_rc != hipSuccess) return check_hip(attr_rc, "lmhead: reserving 128 KB of LDS");
+    hipLaunchKernelGGL(lmhead_partials, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                        static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
                        int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles);
     int rc = check_hip(hipGetLastError(), "lmhead partials launch");

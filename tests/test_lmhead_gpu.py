@@ -22,7 +22,7 @@ def make(n, h, v, seed, w_scale=0.02):
     return hidden, weight, ids
 
 
-@pytest.mark.parametrize("n,h,v", [(1, 32, 1), (5, 64, 7), (300, 256, 1000), (256, 128, 256), (257, 96, 16129),
+@pytest.mark.parametrize("n,h,v", [(1, 64, 1), (5, 64, 7), (300, 256, 1000), (256, 128, 256), (257, 192, 16129),
                                    (64, 4096, 2048), (700, 512, 16385)])
 def test_small_shapes_against_fp64(sampler, n, h, v):
     hidden, weight, ids = make(n, h, v, seed=n + h + v, w_scale=0.2)
@@ -55,7 +55,7 @@ def test_leading_dims_and_invalid_ids(sampler):
     want = O.lmhead_logprob_ref(hidden[keep], weight, ids[keep], dtype=torch.float64)
     assert (flat[keep].double() - want).abs().max().item() <= TOL
     with pytest.raises(ValueError):
-        sampler.fused_linear_logp(hidden[:, :100].contiguous().cuda(), weight[:, :100].contiguous().cuda(), ids.cuda())
+        sampler.fused_linear_logp(hidden[:, :96].contiguous().cuda(), weight[:, :96].contiguous().cuda(), ids.cuda())
 
 
 def test_bit_identical_across_runs_and_row_counts(sampler):
