@@ -26,6 +26,10 @@ for _p in (REPO, REPO / "kernel-align_amd"):
 HBM_PEAK_GBPS = 8000.0
 G, L, V = 256, 512, 128256
 BYTES_PER_TOKEN = 2 * V + 8 + 4
+# HBM traffic of the logprob kernel per token, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
+# program (profiles/logprob_rows_bf16_G256_L512_V128256.txt): 2 x 1,026,607.7 KiB fetched + 258.3 KiB
+# written per 8192-row launch.
+MEASURED_TRAFFIC_PER_TOKEN = (2 * 1026607.7 + 258.3) * 1024 / 8192
 
 
 def log(msg: str) -> None:
@@ -88,6 +92,33 @@ def sampling_latency(sampler, steps: int, warmup: int):
     return out
 
 
+def lmhead_throughput(sampler, iters: int = 3):
+    """Fused lm_head -> logprob on hidden bf16 [32768, 4096] x W bf16 [128256, 4096] (seed 0)."""
+    import torch
+
+    n, h, v = 64 * 512, 4096, V
+    g = torch.Generator(device="cuda").manual_seed(0)
+    hidden = torch.randn(n, h, generator=g, device="cuda").bfloat16()
+    weight = (torch.randn(v, h, generator=g, device="cuda") * 0.02).bfloat16()
+    ids = torch.randint(0, v, (n,), generator=g, device="cuda")
+    for _ in range(2):
+        sampler.fused_linear_logp(hidden, weight, ids)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(iters):
+        out = sampler.fused_linear_logp(hidden, weight, ids)
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / iters
+    tflops = 2.0 * n * h * v / (ms * 1e-3) / 1e12
+    assert bool(torch.isfinite(out).all())
+    return {"config": "hidden bf16 [32768,4096] ~ N(0,1), W bf16 [128256,4096] ~ N(0,0.02^2), seed 0; logits never stored",
+            "ms": ms, "tokens_per_s": n / (ms * 1e-3),
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s",
+                         "frac": tflops / 2500.0, "traffic": None, "kernel": "lmhead_partials"}}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,6 +127,7 @@ def main() -> int:
     ap.add_argument("--cpu-sample-rows", type=int, default=32768,
                     help="rows of the tensor the CPU oracle is timed on (0 = skip)")
     ap.add_argument("--chunk-tokens", type=int, default=None, help="rows per kernel launch")
+    ap.add_argument("--skip-lmhead", action="store_true", help="leave the fused lm_head->logprob figure out")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (torch copy_) three times, so a counter "
                          "run of this command holds a kernel of known traffic to scale FETCH/WRITE_SIZE by")
@@ -175,16 +207,20 @@ def main() -> int:
                    "launches_per_step": launches_per_step, "input_dtype": "bf16", "output_dtype": "f32"},
         "hbm_gbps": n_rows * BYTES_PER_TOKEN / (ms_per_step * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved_gbps / HBM_PEAK_GBPS,
+                     "traffic": rows_per_launch * MEASURED_TRAFFIC_PER_TOKEN,
                      "kernel": "logprob_rows<Bf16,256,4,vec>", "launch_ms": launch_ms,
                      "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
     }
     assert bool(torch.isfinite(out).all()), "non-finite logprob in the timed run"
-    del logits3, ids2
-    result["sampling"] = sampling_latency(sampler, args.steps, args.warmup)
     if args.cpu_sample_rows > 0:
         log("timing the CPU oracle on a sample of the same tensor")
         result["cpu_baseline"] = cpu_baseline(logits, ids, args.cpu_sample_rows)
+    del logits3, ids2, logits, ids
+    torch.cuda.empty_cache()
+    result["sampling"] = sampling_latency(sampler, args.steps, args.warmup)
+    if not args.skip_lmhead:
+        result["fused_lm_head"] = lmhead_throughput(sampler)
     print(json.dumps(result), flush=True)
     return 0
 
