@@ -14,6 +14,8 @@
 //     prefix sums and stops at the first survivor whose inclusive mass exceeds
 //     floor(u * Z_survivors).
 // The row is re-read by every pass; after the first it comes from L2 / MALL.
+#include <stdlib.h>
+
 #include "ka_common.h"
 
 namespace ka {
@@ -117,9 +119,25 @@ __device__ __forceinline__ uint32_t elem_key(typename T::raw_t raw, float temp, 
 // ---------------------------------------------------------------------------
 // Block-wide primitives (1024 threads, fixed exchange pattern)
 // ---------------------------------------------------------------------------
-struct Shared {
+constexpr int CAND_CAP = 1024;  // candidate slots of the top-k fast path (one per thread)
+
+struct Histograms {
     uint32_t cnt[BINS];
     uint64_t mass[BINS];
+};
+struct Candidates {            // 24 KB, same footprint as the histograms
+    uint32_t raw[CAND_CAP];    // element bits as loaded (widened to 32 bits)
+    uint32_t idx[CAND_CAP];
+    uint32_t skey[CAND_CAP];   // scaled keys in (key desc, index asc) order; first used for the thread maxima
+    uint32_t sidx[CAND_CAP];
+    uint64_t w[CAND_CAP];      // integer masses in that order
+};
+
+struct alignas(16) Shared {
+    union {
+        Histograms h;
+        Candidates c;
+    };
     uint64_t wave_u64[S_WAVES];
     uint32_t wave_u32[S_WAVES];
     // broadcast slots
@@ -128,6 +146,8 @@ struct Shared {
     int best_rb;
     uint32_t max_key;
     int64_t hit;
+    uint32_t n_cand, pick_a, pick_b;
+    uint64_t pick_z;
 };
 
 template <typename V> __device__ __forceinline__ V shfl_up_v(V v, int off) { return __shfl_up(v, off, kWave); }
@@ -173,17 +193,16 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, Shared &sh) {
 
 __device__ __forceinline__ void clear_hist(Shared &sh) {
     for (int b = threadIdx.x; b < BINS; b += S_THREADS) {
-        sh.cnt[b] = 0;
-        sh.mass[b] = 0;
+        sh.h.cnt[b] = 0;
+        sh.h.mass[b] = 0;
     }
 }
 
 // ---------------------------------------------------------------------------
-// Row traversal: f(index, key) for every element, any order.
+// Row traversal: f(index, raw element) for every element, any order.
 // ---------------------------------------------------------------------------
 template <typename T, typename F>
-__device__ __forceinline__ void for_each_key(const typename T::raw_t *rp, int vocab, bool vec, float temp,
-                                             bool has_t, F &&f) {
+__device__ __forceinline__ void for_each_raw(const typename T::raw_t *rp, int vocab, bool vec, F &&f) {
     constexpr int EPV = T::kPerVec;
     const int tid = threadIdx.x;
     if (vec) {
@@ -199,20 +218,177 @@ __device__ __forceinline__ void for_each_key(const typename T::raw_t *rp, int vo
             for (int u = 0; u < U; ++u) {
                 const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[u]);
 #pragma unroll
-                for (int j = 0; j < EPV; ++j) f((v + u * S_THREADS) * EPV + j, elem_key<T>(e[j], temp, has_t));
+                for (int j = 0; j < EPV; ++j) f((v + u * S_THREADS) * EPV + j, e[j]);
             }
         }
         for (; v < nvec; v += S_THREADS) {
             const uint4 q = vp[v];
             const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
 #pragma unroll
-            for (int j = 0; j < EPV; ++j) f(v * EPV + j, elem_key<T>(e[j], temp, has_t));
+            for (int j = 0; j < EPV; ++j) f(v * EPV + j, e[j]);
         }
         const int i = nvec * EPV + tid;
-        if (i < vocab) f(i, elem_key<T>(rp[i], temp, has_t));
+        if (i < vocab) f(i, rp[i]);
     } else {
-        for (int i = tid; i < vocab; i += S_THREADS) f(i, elem_key<T>(rp[i], temp, has_t));
+        for (int i = tid; i < vocab; i += S_THREADS) f(i, rp[i]);
     }
+}
+
+// f(index, key of the scaled element).
+template <typename T, typename F>
+__device__ __forceinline__ void for_each_key(const typename T::raw_t *rp, int vocab, bool vec, float temp,
+                                             bool has_t, F &&f) {
+    for_each_raw<T>(rp, vocab, vec, [&](int i, typename T::raw_t raw) { f(i, elem_key<T>(raw, temp, has_t)); });
+}
+
+// Key of the raw (unscaled) element; the scaling x -> round(x / T) is monotone, so order statistics can be
+// located on these keys and only the few candidates need the division.
+template <typename T> __device__ __forceinline__ uint32_t raw_key(typename T::raw_t raw) {
+    return key_of(T::widen(raw));
+}
+template <typename T> __device__ __forceinline__ typename T::raw_t raw_of_key(uint32_t key) {
+    const uint32_t bits = __float_as_uint(value_of(key));
+    if (T::kDtype == KA_DTYPE_BF16) return typename T::raw_t(bits >> 16);
+    if (T::kDtype == KA_DTYPE_F16) {
+        union { _Float16 h; uint16_t u; } c;
+        c.h = _Float16(value_of(key));  // exact: the key came from a widened fp16
+        return typename T::raw_t(c.u);
+    }
+    return typename T::raw_t(bits);
+}
+// Distance between neighbouring representable values in key space.
+template <typename T> __device__ __forceinline__ uint32_t key_step() {
+    return T::kDtype == KA_DTYPE_BF16 ? 0x10000u : (T::kDtype == KA_DTYPE_F16 ? 0x2000u : 1u);
+}
+
+// ---------------------------------------------------------------------------
+// Top-k fast path: everything after the first read of the row happens on a short candidate list in LDS.
+//
+//   1. every lane takes the maximum raw key of its strided share of the row; the top_k-th largest of
+//      those 1024 maxima, t, is a lower bound of the top_k-th largest element;
+//   2. the bound is lowered to the smallest raw key that still scales to the same value as t (ties made
+//      by the rounding of x / T must not be lost), and one more pass collects every element at or above
+//      it: a superset of the top-k survivors, ~top_k + a few entries on ordinary rows;
+//   3. the candidates are scaled, ranked by (key desc, index asc), cut by top-k (ties kept) and top-p on
+//      integer masses, and the draw is taken over the survivors in index order.
+// Returns false (having written nothing) when the candidates do not fit: the radix path then runs.
+// All integer decisions are the same function of the row as in the radix path.
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *rp, int vocab, bool vec, float temp,
+                                          bool has_t, int top_k, bool use_p, float top_p, float u,
+                                          int64_t *out_slot) {
+    const int tid = threadIdx.x;
+    // 1. lane maxima of the raw keys
+    uint32_t lmax = 0;
+    for_each_raw<T>(rp, vocab, vec, [&](int, typename T::raw_t raw) {
+        const uint32_t k = raw_key<T>(raw);
+        lmax = k > lmax ? k : lmax;
+    });
+    __syncthreads();
+    sh.c.skey[tid] = lmax;
+    if (tid == 0) { sh.n_cand = 0; sh.pick_a = 0xffffffffu; sh.hit = -1; }
+    __syncthreads();
+    {   // rank of this lane's maximum among the 1024 (ties broken by lane id); rank top_k-1 is the bound
+        uint32_t rank = 0;
+        for (int j = 0; j < S_THREADS; j += 4) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(&sh.c.skey[j]);
+            rank += (q.x > lmax || (q.x == lmax && j + 0 < tid)) ? 1u : 0u;
+            rank += (q.y > lmax || (q.y == lmax && j + 1 < tid)) ? 1u : 0u;
+            rank += (q.z > lmax || (q.z == lmax && j + 2 < tid)) ? 1u : 0u;
+            rank += (q.w > lmax || (q.w == lmax && j + 3 < tid)) ? 1u : 0u;
+        }
+        if (rank == uint32_t(top_k - 1)) sh.pick_a = lmax;
+    }
+    __syncthreads();
+    uint32_t bound = sh.pick_a;
+    // 2. widen the bound over the raw values that scale to the same value
+    if (has_t) {
+        const uint32_t ty = elem_key<T>(raw_of_key<T>(bound), temp, true);
+        int guard = 0;
+        while (bound >= key_step<T>() && guard < 64) {
+            const uint32_t prev = bound - key_step<T>();
+            if (elem_key<T>(raw_of_key<T>(prev), temp, true) < ty) break;
+            bound = prev;
+            ++guard;
+        }
+        if (guard == 64) return false;  // a huge temperature folds many values together: radix path
+    }
+    for_each_raw<T>(rp, vocab, vec, [&](int i, typename T::raw_t raw) {
+        if (raw_key<T>(raw) >= bound) {
+            const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
+            if (slot < CAND_CAP) {
+                sh.c.raw[slot] = uint32_t(raw);
+                sh.c.idx[slot] = uint32_t(i);
+            }
+        }
+    });
+    __syncthreads();
+    const uint32_t nc = sh.n_cand;
+    if (nc > CAND_CAP) return false;
+    // 3a. scale the candidates and rank them by (key desc, index asc)
+    uint32_t my_key = 0, my_idx = 0;
+    if (tid < int(nc)) {
+        my_key = elem_key<T>(typename T::raw_t(sh.c.raw[tid]), temp, has_t);
+        my_idx = sh.c.idx[tid];
+    }
+    __syncthreads();
+    if (tid < int(nc)) sh.c.raw[tid] = my_key;  // raw[] now holds the scaled keys, unsorted
+    __syncthreads();
+    if (tid < int(nc)) {
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < nc; ++j) {
+            const uint32_t kj = sh.c.raw[j], ij = sh.c.idx[j];
+            rank += (kj > my_key || (kj == my_key && ij < my_idx)) ? 1u : 0u;
+        }
+        sh.c.skey[rank] = my_key;
+        sh.c.sidx[rank] = my_idx;
+    }
+    __syncthreads();
+    // 3b. top-k with ties: survivors are the sorted prefix with key >= key of position top_k - 1
+    const uint32_t kmax = sh.c.skey[0];
+    const float vmax = value_of(kmax);
+    const uint32_t kstar = sh.c.skey[top_k - 1];
+    if (tid < int(nc) && sh.c.skey[tid] >= kstar && (tid + 1 == int(nc) || sh.c.skey[tid + 1] < kstar))
+        sh.pick_b = uint32_t(tid) + 1;
+    __syncthreads();
+    const uint32_t na = sh.pick_b;
+    // 3c. integer masses, exclusive prefix in sorted order, top-p cut
+    uint64_t w = 0;
+    if (tid < int(na)) {
+        const uint32_t k = sh.c.skey[tid];
+        w = weight_fix(k == kmax ? 0.0f : value_of(k) - vmax);
+        sh.c.w[tid] = w;
+    }
+    uint64_t z_topk;
+    const uint64_t before = block_excl_scan<uint64_t>(w, sh.wave_u64, &z_topk);
+    uint32_t nb = na;
+    uint64_t z_kept = z_topk;
+    if (use_p) {
+        const uint64_t theta = floor_scale(top_p, z_topk);
+        const bool kept = tid < int(na) && before <= theta;
+        // `before` is non-decreasing along the sorted order, so the survivors are a prefix; its last lane
+        // publishes the count and the surviving mass
+        const uint64_t next_before = before + w;
+        if (kept && (tid + 1 == int(na) || next_before > theta)) {
+            sh.pick_a = uint32_t(tid) + 1;
+            sh.pick_z = next_before;
+        }
+        __syncthreads();
+        nb = sh.pick_a;
+        z_kept = sh.pick_z;
+    }
+    // 3d. draw: inclusive mass over the survivors in index order; the first index above floor(u * Z) wins
+    const uint64_t tau = floor_scale(u, z_kept);
+    if (tid < int(nb)) {
+        const uint32_t mine = sh.c.sidx[tid];
+        uint64_t cum = 0;
+        for (uint32_t j = 0; j < nb; ++j) cum += sh.c.sidx[j] <= mine ? sh.c.w[j] : 0ull;
+        if (cum > tau) atomicMin(reinterpret_cast<unsigned long long *>(&sh.hit), (unsigned long long)mine);
+    }
+    __syncthreads();
+    if (tid == 0) *out_slot = sh.hit;
+    return true;
 }
 
 // ---------------------------------------------------------------------------
@@ -223,7 +399,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                                                          int vocab, int64_t row_stride, float temp,
                                                          int top_k, float top_p,
                                                          const float *__restrict__ uniforms,
-                                                         int64_t *__restrict__ out, int vec) {
+                                                         int64_t *__restrict__ out, int vec, int no_fast) {
     constexpr int EPV = T::kPerVec;
     constexpr int LEVELS = Round<T>::kLevels;
     __shared__ Shared sh;
@@ -234,13 +410,22 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     const bool use_k = top_k > 0 && top_k < vocab;
     const bool use_p = top_p < 1.0f;
 
+    float u = uniforms[row];
+    if (!(u >= 0.0f)) u = 0.0f;
+    if (u >= 1.0f) u = __uint_as_float(0x3f7fffffu);
+
+    if (use_k && top_k <= S_THREADS && !no_fast) {
+        if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row)) return;
+        __syncthreads();
+    }
+
     // ---- pass 0: row maximum and the level-0 count histogram --------------------------
     clear_hist(sh);
     __syncthreads();
     uint32_t kmax = 0;
     for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
         kmax = key > kmax ? key : kmax;
-        if (use_k) atomicAdd(&sh.cnt[key >> 21], 1u);
+        if (use_k) atomicAdd(&sh.h.cnt[key >> 21], 1u);
     });
     kmax = block_max_u32(kmax, sh);  // barriers inside also publish the histogram
     const float vmax = value_of(kmax);
@@ -259,14 +444,14 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                 __syncthreads();
                 const int pshift = level_shift<T>(level - 1);
                 for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
-                    if ((key >> pshift) == prefix) atomicAdd(&sh.cnt[(key >> shift) & (nb - 1)], 1u);
+                    if ((key >> pshift) == prefix) atomicAdd(&sh.h.cnt[(key >> shift) & (nb - 1)], 1u);
                 });
                 __syncthreads();
             }
             // thread t owns the bins 2t and 2t+1 counted from the top
             const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
-            const uint32_t c0 = rb0 < int(nb) ? sh.cnt[nb - 1 - rb0] : 0u;
-            const uint32_t c1 = rb1 < int(nb) ? sh.cnt[nb - 1 - rb1] : 0u;
+            const uint32_t c0 = rb0 < int(nb) ? sh.h.cnt[nb - 1 - rb0] : 0u;
+            const uint32_t c1 = rb1 < int(nb) ? sh.h.cnt[nb - 1 - rb1] : 0u;
             uint32_t total;
             const uint32_t excl = block_excl_scan<uint32_t>(c0 + c1, sh.wave_u32, &total);
             if (excl < rank && rank <= excl + c0) {
@@ -293,8 +478,8 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
             const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
             zpart += w;
             if (use_p) {
-                atomicAdd(reinterpret_cast<unsigned long long *>(&sh.mass[key >> 21]), (unsigned long long)w);
-                atomicAdd(&sh.cnt[key >> 21], 1u);
+                atomicAdd(reinterpret_cast<unsigned long long *>(&sh.h.mass[key >> 21]), (unsigned long long)w);
+                atomicAdd(&sh.h.cnt[key >> 21], 1u);
             }
         }
     });
@@ -324,17 +509,17 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                         const float y = value_of(key);
                         const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
                         const uint32_t d = (key >> shift) & (nb - 1);
-                        atomicAdd(reinterpret_cast<unsigned long long *>(&sh.mass[d]), (unsigned long long)w);
-                        atomicAdd(&sh.cnt[d], 1u);
+                        atomicAdd(reinterpret_cast<unsigned long long *>(&sh.h.mass[d]), (unsigned long long)w);
+                        atomicAdd(&sh.h.cnt[d], 1u);
                     }
                 });
                 __syncthreads();
             }
             const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
-            const uint64_t m0 = rb0 < int(nb) ? sh.mass[nb - 1 - rb0] : 0ull;
-            const uint64_t m1 = rb1 < int(nb) ? sh.mass[nb - 1 - rb1] : 0ull;
-            const uint32_t c0 = rb0 < int(nb) ? sh.cnt[nb - 1 - rb0] : 0u;
-            const uint32_t c1 = rb1 < int(nb) ? sh.cnt[nb - 1 - rb1] : 0u;
+            const uint64_t m0 = rb0 < int(nb) ? sh.h.mass[nb - 1 - rb0] : 0ull;
+            const uint64_t m1 = rb1 < int(nb) ? sh.h.mass[nb - 1 - rb1] : 0ull;
+            const uint32_t c0 = rb0 < int(nb) ? sh.h.cnt[nb - 1 - rb0] : 0u;
+            const uint32_t c1 = rb1 < int(nb) ? sh.h.cnt[nb - 1 - rb1] : 0u;
             uint64_t total;
             const uint64_t excl = block_excl_scan<uint64_t>(m0 + m1, sh.wave_u64, &total);
             if (tid == 0) sh.best_rb = -1;
@@ -367,9 +552,6 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     }
 
     // ---- draw: first survivor, in index order, whose inclusive mass exceeds floor(u * Z) ----
-    float u = uniforms[row];
-    if (!(u >= 0.0f)) u = 0.0f;
-    if (u >= 1.0f) u = __uint_as_float(0x3f7fffffu);
     const uint64_t tau = floor_scale(u, z_kept);
     const bool track_ties = r_cut != 0xffffffffu;
     if (tid == 0) sh.hit = -1;
@@ -427,6 +609,12 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (tid == 0) out[row] = sh.hit;
 }
 
+// KA_SAMPLE_RADIX_ONLY=1 switches the top-k fast path off (the tests use it to run both paths on every case).
+inline bool force_radix_path() {
+    const char *e = getenv("KA_SAMPLE_RADIX_ONLY");
+    return e != nullptr && e[0] == '1';
+}
+
 template <typename T>
 int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride, float temperature,
            int32_t top_k, float top_p, const float *uniforms, int64_t *out_ids, void *workspace,
@@ -451,7 +639,7 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
     hipLaunchKernelGGL((sample_rows<T>), dim3(unsigned(batch)), dim3(S_THREADS), 0,
                        static_cast<hipStream_t>(hip_stream),
                        static_cast<const typename T::raw_t *>(logits), int(vocab), row_stride, temperature,
-                       int(top_k), top_p, uniforms, out_ids, aligned ? 1 : 0);
+                       int(top_k), top_p, uniforms, out_ids, aligned ? 1 : 0, force_radix_path() ? 1 : 0);
     return check_hip(hipGetLastError(), "sample launch");
 }
 

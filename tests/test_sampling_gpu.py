@@ -149,3 +149,32 @@ def test_invalid_arguments_raise(sampler):
         sampler.sample(logits.cpu(), top_k=5)
     with pytest.raises(ValueError):
         sampler.sample(logits, uniforms=torch.zeros(3, device="cuda"))
+
+
+def test_fast_and_radix_paths_are_the_same_function(sampler, monkeypatch):
+    """top_k <= 1024 normally runs on a candidate list in LDS; KA_SAMPLE_RADIX_ONLY=1 forces the radix
+    descents.  Both must return the same ids (and both are checked against the oracle elsewhere)."""
+    g = torch.Generator().manual_seed(31)
+    cases = []
+    for dtype in DTYPES:
+        cases.append((torch.randn(32, 50000, generator=g).mul(3).to(dtype), 50, 0.9, 0.7))
+        cases.append((((torch.randn(32, 6000, generator=g) * 8).round() / 4).to(dtype), 7, 0.6, 1.0))   # heavy ties
+        cases.append((torch.randn(32, 3000, generator=g).to(dtype), 1000, None, 1.9))
+        cases.append((torch.zeros(4, 128256).to(dtype), 50, 0.3, 0.7))                                  # overflow -> radix
+    for logits, k, p, temp in cases:
+        u = torch.rand(logits.shape[0], generator=g)
+        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
+        fast = run(sampler, logits, u, k, p, temp)
+        monkeypatch.setenv("KA_SAMPLE_RADIX_ONLY", "1")
+        radix = run(sampler, logits, u, k, p, temp)
+        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
+        assert torch.equal(fast, radix)
+        assert torch.equal(fast, exact.sample(logits, temp, k, p, u))
+
+
+def test_huge_temperature_folds_values_together(sampler):
+    g = torch.Generator().manual_seed(32)
+    logits = (torch.randn(8, 20000, generator=g) * 3).bfloat16()
+    u = torch.rand(8, generator=g)
+    for temp in (1e3, 1e30, 3e38):
+        check_exact(sampler, logits, u, 50, 0.9, temp)
