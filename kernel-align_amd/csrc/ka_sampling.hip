@@ -33,8 +33,15 @@ __device__ __forceinline__ uint32_t key_of(float y) {
     const uint32_t b = __float_as_uint(y);
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
-__device__ __forceinline__ float value_of(uint32_t key) {
-    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+// Keys of 16-bit dtypes keep only their significant top bits (a widened bf16 has 16, a widened fp16 19):
+// negative values would otherwise carry ones in the unused low bits, and a key rebuilt from radix digits
+// would not compare equal to the key of the element it came from.
+template <typename T> __device__ __forceinline__ constexpr uint32_t key_mask() {
+    return T::kDtype == KA_DTYPE_BF16 ? 0xffff0000u : (T::kDtype == KA_DTYPE_F16 ? 0xffffe000u : 0xffffffffu);
+}
+template <typename T> __device__ __forceinline__ uint32_t masked_key(float y) { return key_of(y) & key_mask<T>(); }
+template <typename T> __device__ __forceinline__ float value_of(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : (~key & key_mask<T>()));
 }
 
 // W(d) = trunc(2^40 * exp(d)), d <= 0.  Separate IEEE multiplies and adds (the
@@ -113,7 +120,7 @@ __device__ __forceinline__ uint32_t elem_key(typename T::raw_t raw, float temp, 
     float y = T::widen(raw);
     if (has_t) y = Round<T>::apply(y / temp);
     y = (y == 0.0f) ? 0.0f : y;
-    return key_of(y);
+    return masked_key<T>(y);
 }
 
 // ---------------------------------------------------------------------------
@@ -191,6 +198,31 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, Shared &sh) {
     return r;
 }
 
+// Finds the bin of sh.h.cnt[0 .. nb) that holds the rank-th largest entry (rank is 1-based, bins are ordered
+// by digit, larger digit = larger keys).  Returns the digit; *above = entries in higher bins, *count =
+// entries in the bin.  Every thread must call it; it contains barriers.
+__device__ __forceinline__ uint32_t select_count_bin(Shared &sh, uint32_t nb, uint32_t rank, uint32_t *above,
+                                                     uint32_t *count) {
+    const int tid = threadIdx.x;
+    // thread t owns the bins 2t and 2t+1 counted from the top
+    const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
+    const uint32_t c0 = rb0 < int(nb) ? sh.h.cnt[nb - 1 - rb0] : 0u;
+    const uint32_t c1 = rb1 < int(nb) ? sh.h.cnt[nb - 1 - rb1] : 0u;
+    uint32_t total;
+    const uint32_t excl = block_excl_scan<uint32_t>(c0 + c1, sh.wave_u32, &total);
+    if (excl < rank && rank <= excl + c0) {
+        sh.sel_digit = nb - 1 - rb0; sh.sel_above = excl; sh.sel_count = c0;
+    } else if (excl + c0 < rank && rank <= excl + c0 + c1) {
+        sh.sel_digit = nb - 1 - rb1; sh.sel_above = excl + c0; sh.sel_count = c1;
+    }
+    __syncthreads();
+    const uint32_t digit = sh.sel_digit;
+    *above = sh.sel_above;
+    *count = sh.sel_count;
+    __syncthreads();
+    return digit;
+}
+
 __device__ __forceinline__ void clear_hist(Shared &sh) {
     for (int b = threadIdx.x; b < BINS; b += S_THREADS) {
         sh.h.cnt[b] = 0;
@@ -201,14 +233,13 @@ __device__ __forceinline__ void clear_hist(Shared &sh) {
 // ---------------------------------------------------------------------------
 // Row traversal: f(index, raw element) for every element, any order.
 // ---------------------------------------------------------------------------
-template <typename T, typename F>
+template <typename T, int U = 4, typename F>
 __device__ __forceinline__ void for_each_raw(const typename T::raw_t *rp, int vocab, bool vec, F &&f) {
     constexpr int EPV = T::kPerVec;
     const int tid = threadIdx.x;
     if (vec) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
         const int nvec = vocab / EPV;
-        constexpr int U = 4;
         int v = tid;
         for (; v + (U - 1) * S_THREADS < nvec; v += U * S_THREADS) {
             uint4 q[U];
@@ -244,14 +275,14 @@ __device__ __forceinline__ void for_each_key(const typename T::raw_t *rp, int vo
 // Key of the raw (unscaled) element; the scaling x -> round(x / T) is monotone, so order statistics can be
 // located on these keys and only the few candidates need the division.
 template <typename T> __device__ __forceinline__ uint32_t raw_key(typename T::raw_t raw) {
-    return key_of(T::widen(raw));
+    return masked_key<T>(T::widen(raw));
 }
 template <typename T> __device__ __forceinline__ typename T::raw_t raw_of_key(uint32_t key) {
-    const uint32_t bits = __float_as_uint(value_of(key));
+    const uint32_t bits = __float_as_uint(value_of<T>(key));
     if (T::kDtype == KA_DTYPE_BF16) return typename T::raw_t(bits >> 16);
     if (T::kDtype == KA_DTYPE_F16) {
         union { _Float16 h; uint16_t u; } c;
-        c.h = _Float16(value_of(key));  // exact: the key came from a widened fp16
+        c.h = _Float16(value_of<T>(key));  // exact: the key came from a widened fp16
         return typename T::raw_t(c.u);
     }
     return typename T::raw_t(bits);
@@ -279,29 +310,33 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                                           bool has_t, int top_k, bool use_p, float top_p, float u,
                                           int64_t *out_slot) {
     const int tid = threadIdx.x;
-    // 1. lane maxima of the raw keys
-    uint32_t lmax = 0;
-    for_each_raw<T>(rp, vocab, vec, [&](int, typename T::raw_t raw) {
-        const uint32_t k = raw_key<T>(raw);
-        lmax = k > lmax ? k : lmax;
-    });
-    __syncthreads();
-    sh.c.skey[tid] = lmax;
-    if (tid == 0) { sh.n_cand = 0; sh.pick_a = 0xffffffffu; sh.hit = -1; }
-    __syncthreads();
-    {   // rank of this lane's maximum among the 1024 (ties broken by lane id); rank top_k-1 is the bound
-        uint32_t rank = 0;
-        for (int j = 0; j < S_THREADS; j += 4) {
-            const uint4 q = *reinterpret_cast<const uint4 *>(&sh.c.skey[j]);
-            rank += (q.x > lmax || (q.x == lmax && j + 0 < tid)) ? 1u : 0u;
-            rank += (q.y > lmax || (q.y == lmax && j + 1 < tid)) ? 1u : 0u;
-            rank += (q.z > lmax || (q.z == lmax && j + 2 < tid)) ? 1u : 0u;
-            rank += (q.w > lmax || (q.w == lmax && j + 3 < tid)) ? 1u : 0u;
+    // 1. lane maxima of the raw values (float max: one convert and half a v_max3 per element; which of
+    //    -0 / +0 it returns does not matter, any lower bound of the top_k-th element will do)
+    float lmaxf = -__builtin_inff();
+    for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) { lmaxf = fmaxf(lmaxf, T::widen(raw)); });
+    const uint32_t lmax = masked_key<T>(lmaxf);
+    // the top_k-th largest of the 1024 lane maxima, by the same MSB-first descent over count histograms
+    uint32_t bound = 0;
+    {
+        uint32_t rank = uint32_t(top_k), prefix = 0;
+        for (int level = 0; level < Round<T>::kLevels; ++level) {
+            const int shift = level_shift<T>(level), bits = level_bits<T>(level);
+            const uint32_t nb = 1u << bits;
+            __syncthreads();
+            for (int b = tid; b < int(nb); b += S_THREADS) sh.h.cnt[b] = 0;
+            __syncthreads();
+            if (level == 0 || (lmax >> level_shift<T>(level - 1)) == prefix)
+                atomicAdd(&sh.h.cnt[(lmax >> shift) & (nb - 1)], 1u);
+            __syncthreads();
+            uint32_t above, count;
+            const uint32_t digit = select_count_bin(sh, nb, rank, &above, &count);
+            prefix = (prefix << bits) | digit;
+            rank -= above;
         }
-        if (rank == uint32_t(top_k - 1)) sh.pick_a = lmax;
+        bound = prefix << level_shift<T>(Round<T>::kLevels - 1);
     }
+    if (tid == 0) { sh.n_cand = 0; sh.hit = -1; }
     __syncthreads();
-    uint32_t bound = sh.pick_a;
     // 2. widen the bound over the raw values that scale to the same value
     if (has_t) {
         const uint32_t ty = elem_key<T>(raw_of_key<T>(bound), temp, true);
@@ -314,8 +349,9 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         }
         if (guard == 64) return false;  // a huge temperature folds many values together: radix path
     }
-    for_each_raw<T>(rp, vocab, vec, [&](int i, typename T::raw_t raw) {
-        if (raw_key<T>(raw) >= bound) {
+    const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
+    for_each_raw<T, 8>(rp, vocab, vec, [&](int i, typename T::raw_t raw) {
+        if (T::widen(raw) >= boundf) {
             const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
             if (slot < CAND_CAP) {
                 sh.c.raw[slot] = uint32_t(raw);
@@ -334,8 +370,30 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     }
     __syncthreads();
     if (tid < int(nc)) sh.c.raw[tid] = my_key;  // raw[] now holds the scaled keys, unsorted
+    uint32_t *const rank_of = reinterpret_cast<uint32_t *>(sh.c.w);  // scratch until the masses are written
+    if (tid < kWave) rank_of[tid] = 0;
     __syncthreads();
-    if (tid < int(nc)) {
+    if (nc <= kWave) {
+        // short list (the ordinary case): candidate i = lane, wavefront w counts against entries 4w .. 4w+3
+        const int i = tid & (kWave - 1), j0 = (tid / kWave) * 4;
+        if (i < int(nc) && j0 < int(nc)) {
+            const uint32_t ki = sh.c.raw[i], ii = sh.c.idx[i];
+            uint32_t part = 0;
+#pragma unroll
+            for (int j = j0; j < j0 + 4; ++j)
+                if (j < int(nc)) {
+                    const uint32_t kj = sh.c.raw[j], ij = sh.c.idx[j];
+                    part += (kj > ki || (kj == ki && ij < ii)) ? 1u : 0u;
+                }
+            if (part) atomicAdd(&rank_of[i], part);
+        }
+        __syncthreads();
+        if (tid < int(nc)) {
+            const uint32_t rank = rank_of[tid];
+            sh.c.skey[rank] = my_key;
+            sh.c.sidx[rank] = my_idx;
+        }
+    } else if (tid < int(nc)) {
         uint32_t rank = 0;
         for (uint32_t j = 0; j < nc; ++j) {
             const uint32_t kj = sh.c.raw[j], ij = sh.c.idx[j];
@@ -347,7 +405,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     __syncthreads();
     // 3b. top-k with ties: survivors are the sorted prefix with key >= key of position top_k - 1
     const uint32_t kmax = sh.c.skey[0];
-    const float vmax = value_of(kmax);
+    const float vmax = value_of<T>(kmax);
     const uint32_t kstar = sh.c.skey[top_k - 1];
     if (tid < int(nc) && sh.c.skey[tid] >= kstar && (tid + 1 == int(nc) || sh.c.skey[tid + 1] < kstar))
         sh.pick_b = uint32_t(tid) + 1;
@@ -357,7 +415,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     uint64_t w = 0;
     if (tid < int(na)) {
         const uint32_t k = sh.c.skey[tid];
-        w = weight_fix(k == kmax ? 0.0f : value_of(k) - vmax);
+        w = weight_fix(k == kmax ? 0.0f : value_of<T>(k) - vmax);
         sh.c.w[tid] = w;
     }
     uint64_t z_topk;
@@ -428,7 +486,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
         if (use_k) atomicAdd(&sh.h.cnt[key >> 21], 1u);
     });
     kmax = block_max_u32(kmax, sh);  // barriers inside also publish the histogram
-    const float vmax = value_of(kmax);
+    const float vmax = value_of<T>(kmax);
 
     // ---- top-k: MSB-first descent to the k-th largest key --------------------------------
     uint32_t kstar = 0;      // keep key >= kstar
@@ -448,22 +506,10 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                 });
                 __syncthreads();
             }
-            // thread t owns the bins 2t and 2t+1 counted from the top
-            const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
-            const uint32_t c0 = rb0 < int(nb) ? sh.h.cnt[nb - 1 - rb0] : 0u;
-            const uint32_t c1 = rb1 < int(nb) ? sh.h.cnt[nb - 1 - rb1] : 0u;
-            uint32_t total;
-            const uint32_t excl = block_excl_scan<uint32_t>(c0 + c1, sh.wave_u32, &total);
-            if (excl < rank && rank <= excl + c0) {
-                sh.sel_digit = nb - 1 - rb0; sh.sel_above = excl; sh.sel_count = c0;
-            } else if (excl + c0 < rank && rank <= excl + c0 + c1) {
-                sh.sel_digit = nb - 1 - rb1; sh.sel_above = excl + c0; sh.sel_count = c1;
-            }
-            __syncthreads();
-            prefix = (prefix << bits) | sh.sel_digit;
-            rank -= sh.sel_above;
-            n_eq_kstar = sh.sel_count;
-            __syncthreads();
+            uint32_t above;
+            const uint32_t digit = select_count_bin(sh, nb, rank, &above, &n_eq_kstar);
+            prefix = (prefix << bits) | digit;
+            rank -= above;
         }
         kstar = prefix << level_shift<T>(LEVELS - 1);
     }
@@ -474,7 +520,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     uint64_t zpart = 0;
     for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
         if (key >= kstar) {
-            const float y = value_of(key);
+            const float y = value_of<T>(key);
             const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
             zpart += w;
             if (use_p) {
@@ -506,7 +552,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                 const int pshift = level_shift<T>(level - 1);
                 for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
                     if (key >= kstar && (key >> pshift) == prefix) {
-                        const float y = value_of(key);
+                        const float y = value_of<T>(key);
                         const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
                         const uint32_t d = (key >> shift) & (nb - 1);
                         atomicAdd(reinterpret_cast<unsigned long long *>(&sh.h.mass[d]), (unsigned long long)w);
@@ -589,7 +635,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                 if (keys[j] > kcut) member = true;
                 else if (keys[j] == kcut && keys[j] >= kstar) member = !track_ties || (tie_rank++ < r_cut);
             }
-            w[j] = member ? weight_fix(keys[j] == kmax ? 0.0f : value_of(keys[j]) - vmax) : 0ull;
+            w[j] = member ? weight_fix(keys[j] == kmax ? 0.0f : value_of<T>(keys[j]) - vmax) : 0ull;
             msum += w[j];
         }
         uint64_t tot;

@@ -67,11 +67,16 @@ def test_heavy_ties_and_degenerate_rows(sampler, dtype, k, p, temp):
     logits[4, :] = 0.0
     logits[4, 100:200] = -0.0                # signed zeros are one value
     logits[5, 5] = 30.0                      # one dominant entry: everything else has mass ~0
+    logits[6, :] = -2.0                      # all equal and negative: the cut key is a negative value
+    logits[7] = -logits[7].abs() - 1.0       # only negative values, coarse grid: negative ties at k-th value and cut
+    logits[8, :] = -math.inf
+    logits[8, 10:40] = -7.5                  # few finite negative entries over a -inf background
     check_exact(sampler, logits, u, k, p, temp)
 
 
-def test_all_equal_llama_row_cut_inside_tie_group(sampler):
-    logits = torch.zeros(4, 128256, dtype=torch.bfloat16)
+@pytest.mark.parametrize("value", [0.0, -3.0, 2.5])
+def test_all_equal_llama_row_cut_inside_tie_group(sampler, value):
+    logits = torch.full((4, 128256), value, dtype=torch.bfloat16)
     u = torch.tensor([0.0, 0.25, 0.5, 0.999])
     got = check_exact(sampler, logits, u, 50, 0.3, 0.7)
     kept = math.floor(float(torch.tensor(0.3, dtype=torch.float32)) * 128256) + 1
