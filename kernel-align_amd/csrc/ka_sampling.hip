@@ -312,8 +312,34 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     const int tid = threadIdx.x;
     // 1. lane maxima of the raw values (float max: one convert and half a v_max3 per element; which of
     //    -0 / +0 it returns does not matter, any lower bound of the top_k-th element will do)
+    //    When the row fits (16-byte aligned, at most 16 vectors per lane: 131,072 bf16 entries) it is kept in
+    //    registers, so that the collection pass below reads nothing from memory.
+    constexpr int EPV = T::kPerVec;
+    constexpr int RES_VECS = 16;
+    const int nvec = vocab / EPV;
+    const bool resident = vec && T::kDtype == KA_DTYPE_BF16 && nvec <= RES_VECS * S_THREADS;
+    uint4 held[RES_VECS];
     float lmaxf = -__builtin_inff();
-    for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) { lmaxf = fmaxf(lmaxf, T::widen(raw)); });
+    if (resident) {
+        const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+#pragma unroll
+        for (int r = 0; r < RES_VECS; ++r) {
+            const int v = tid + r * S_THREADS;
+            held[r] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < RES_VECS; ++r) {
+            if (tid + r * S_THREADS < nvec) {
+                const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&held[r]);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) lmaxf = fmaxf(lmaxf, T::widen(e[j]));
+            }
+        }
+        const int i = nvec * EPV + tid;  // ragged tail of the row
+        if (i < vocab) lmaxf = fmaxf(lmaxf, T::widen(rp[i]));
+    } else {
+        for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) { lmaxf = fmaxf(lmaxf, T::widen(raw)); });
+    }
     const uint32_t lmax = masked_key<T>(lmaxf);
     // the top_k-th largest of the 1024 lane maxima, by the same MSB-first descent over count histograms
     uint32_t bound = 0;
@@ -350,7 +376,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         if (guard == 64) return false;  // a huge temperature folds many values together: radix path
     }
     const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
-    for_each_raw<T, 8>(rp, vocab, vec, [&](int i, typename T::raw_t raw) {
+    auto collect = [&](int i, typename T::raw_t raw) {
         if (T::widen(raw) >= boundf) {
             const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
             if (slot < CAND_CAP) {
@@ -358,7 +384,27 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                 sh.c.idx[slot] = uint32_t(i);
             }
         }
-    });
+    };
+    if (resident) {
+#pragma unroll
+        for (int r = 0; r < RES_VECS; ++r) {
+            const int v = tid + r * S_THREADS;
+            if (v < nvec) {
+                const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&held[r]);
+                float vm = T::widen(e[0]);
+#pragma unroll
+                for (int j = 1; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
+                if (vm >= boundf) {  // rare: about top_k vectors of the whole row hold a candidate
+#pragma unroll
+                    for (int j = 0; j < EPV; ++j) collect(v * EPV + j, e[j]);
+                }
+            }
+        }
+        const int i = nvec * EPV + tid;
+        if (i < vocab) collect(i, rp[i]);
+    } else {
+        for_each_raw<T, 8>(rp, vocab, vec, collect);
+    }
     __syncthreads();
     const uint32_t nc = sh.n_cand;
     if (nc > CAND_CAP) return false;
