@@ -55,7 +55,7 @@ def test_leading_dims_and_invalid_ids(sampler):
     want = O.lmhead_logprob_ref(hidden[keep], weight, ids[keep], dtype=torch.float64)
     assert (flat[keep].double() - want).abs().max().item() <= TOL
     with pytest.raises(ValueError):
-        sampler.fused_linear_logp(hidden[:, :96].contiguous().cuda(), weight[:, :96].contiguous().cuda(), ids.cuda())
+        sampler.fused_linear_logp(hidden[:, :80].contiguous().cuda(), weight[:, :80].contiguous().cuda(), ids.cuda())
 
 
 def test_bit_identical_across_runs_and_row_counts(sampler):
