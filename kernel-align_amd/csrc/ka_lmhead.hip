@@ -4,10 +4,10 @@
 // Tiling (gfx950, wave64, v_mfma_f32_32x32x16_bf16):
 //   * a workgroup of 4 wavefronts owns 256 tokens and walks a range of 256-row
 //     vocabulary tiles; per tile it runs a K loop over the hidden dimension in
-//     slabs of 32; the W slab [256 x 32] and the hidden slab [256 x 32] go from
-//     global memory straight into XOR-swizzled LDS (global_load_lds_dwordx4, no
-//     register staging) through a ring of four 32 KB stages, so copies run three
-//     slabs ahead of the MFMAs; one barrier per slab;
+//     slabs of 64 (one cache line per row); the W slab [256 x 64] and the hidden
+//     slab [256 x 64] go from global memory straight into XOR-swizzled LDS
+//     (global_load_lds_dwordx4, no register staging), two stages of 64 KB, one
+//     barrier per slab; fragment reads run one k-step ahead of the MFMAs;
 //   * the MFMA "A" operand is W (rows of the result = vocabulary entries) and
 //     "B" is hidden (columns = tokens), so every lane's 64 accumulators of one
 //     32-column block belong to ONE token: the online max / sum-of-exp update
@@ -26,11 +26,10 @@ namespace {
 
 constexpr int LM_BM = 256;      // vocabulary rows per tile
 constexpr int LM_BN = 256;      // tokens per workgroup
-constexpr int LM_BK = 32;       // hidden slab
-constexpr int LM_STAGES = 4;    // LDS ring: the slab in use plus three in flight
-constexpr int LM_STAGE_ELEMS = (LM_BM + LM_BN) * LM_BK;  // bf16 elements per LDS stage (32 KB)
+constexpr int LM_BK = 64;       // hidden slab: one 128-byte line per row
+constexpr int LM_STAGES = 2;    // LDS: the slab in use and the slab in flight
+constexpr int LM_STAGE_ELEMS = (LM_BM + LM_BN) * LM_BK;  // bf16 elements per LDS stage (64 KB)
 constexpr int LM_LDS_BYTES = LM_STAGES * LM_STAGE_ELEMS * 2;
-constexpr int LM_COPIES_PER_SLAB = 8;  // global->LDS instructions per wavefront and slab
 constexpr int LM_THREADS = 256;
 constexpr int LM_TILES_PER_SPLIT = 63;
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -47,12 +46,11 @@ struct Partial {
     float pad;
 };
 
-// LDS slab: 256 rows x 32 bf16 (64 B per row = four 16-byte chunks; two rows share a 128-byte bank line).
-// A fragment read (ds_read_b128) has lane l fetch row l % 32 at logical chunk 2*kk + l / 32.  The chunk
-// index is XOR-swizzled with swz(row) = (row & 2) | ((row >> 2) & 1), so that eight consecutive rows at one
-// logical chunk, and four consecutive rows at two neighbouring chunks, each touch eight different
-// 16-byte columns.
-__device__ __forceinline__ int swz(int row) { return (row & 2) | ((row >> 2) & 1); }
+// LDS slab: 256 rows x 64 bf16 (128 B per row = eight 16-byte chunks).  A fragment read (ds_read_b128) has
+// lane l fetch row l % 32 at logical chunk 2*kk + l / 32.  The chunk index is XOR-swizzled with
+// swz(row) = (row >> 1) & 7; measured with a ds_read_b128 micro-benchmark on gfx950 this pattern reads at
+// the same rate as a contiguous one, while (row & 7) and an unswizzled slab cost 1.5x and 4.5x.
+__device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int slab_offset(int row, int chunk) {
     return row * LM_BK + ((chunk ^ swz(row)) << 3);  // in bf16 elements
 }
@@ -101,97 +99,60 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     }
 
     // Global -> LDS copies.  One global_load_lds_dwordx4 moves 16 B per lane to LDS base + 16 * lane,
-    // i.e. one wavefront fills sixteen consecutive 64-byte rows; instruction j of wavefront w covers rows
-    // (4j + w) * 16 .. + 15.  Lane l therefore fetches row (4j + w) * 16 + l / 4 and, because the slab is
-    // swizzled, the logical chunk (l % 4) ^ swz(l / 4).  Row offsets are 32-bit byte offsets from a
-    // wavefront-uniform base (the host checks that both matrices are smaller than 4 GiB).
-    const int cp_row = wave * 16 + (lane >> 2);                // + 64 * j
-    const int cp_chunk = (lane & 3) ^ swz(lane >> 2);
-    uint32_t hoff[4];
+    // i.e. one wavefront fills eight consecutive 128-byte rows (eight full cache lines); instruction j of
+    // wavefront w covers rows (4j + w) * 8 .. + 7.  Lane l therefore fetches row (4j + w) * 8 + l / 8 and,
+    // because the slab is swizzled, the logical chunk (l % 8) ^ swz(row).  Row offsets are 32-bit byte
+    // offsets from a wavefront-uniform base (the host checks that both matrices are smaller than 4 GiB).
+    const int cp_row = wave * 8 + (lane >> 3);                 // + 32 * j
+    uint32_t hoff[8];
+    int cp_chunk[8];                                           // swz depends on bits 1..3 of the row: on j too
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-        hoff[j] = uint32_t(min(tok0 + cp_row + 64 * j, n_rows - 1)) * uint32_t(hdim) * 2u + cp_chunk * 16u;
-    const int wave_lds = __builtin_amdgcn_readfirstlane(wave) * 512;  // bf16 elements: 16 rows of 32
+    for (int j = 0; j < 8; ++j) {
+        cp_chunk[j] = (lane & 7) ^ swz(cp_row + 32 * j);
+        hoff[j] = uint32_t(min(tok0 + cp_row + 32 * j, n_rows - 1)) * uint32_t(hdim) * 2u + cp_chunk[j] * 16u;
+    }
+    const int wave_lds = __builtin_amdgcn_readfirstlane(wave) * 512;  // bf16 elements: 8 rows of 64
     const char *const wbytes = reinterpret_cast<const char *>(weight);
     const char *const hbytes = reinterpret_cast<const char *>(hidden);
 
-    // Requests copy j (0..7: W rows for even j, hidden rows for odd j) of slab (vt_, kt_) into stage stage_.
-#define LM_ISSUE_ONE(j_, vt_, kt_, stage_)                                                                   \
+    // Requests copy c (0..15: W rows for even c, hidden rows for odd c) of slab (vt_, kt_) into stage stage_.
+#define LM_ISSUE_ONE(c_, vt_, kt_, stage_)                                                                   \
     do {                                                                                                     \
         const size_t kb_ = size_t(kt_) * (LM_BK * 2);                                                        \
-        uint16_t *sa_ = lds + (stage_) * LM_STAGE_ELEMS + wave_lds + ((j_) >> 1) * 2048;                      \
-        if (((j_) & 1) == 0) {                                                                               \
-            const uint32_t woff_ = uint32_t(min((vt_) * LM_BM + cp_row + 64 * ((j_) >> 1), vocab - 1)) * uint32_t(hdim) * 2u + cp_chunk * 16u; \
+        uint16_t *sa_ = lds + (stage_) * LM_STAGE_ELEMS + wave_lds + ((c_) >> 1) * 2048;                      \
+        if (((c_) & 1) == 0) {                                                                               \
+            const uint32_t woff_ = uint32_t(min((vt_) * LM_BM + cp_row + 32 * ((c_) >> 1), vocab - 1)) * uint32_t(hdim) * 2u + cp_chunk[(c_) >> 1] * 16u; \
             __builtin_amdgcn_global_load_lds(wbytes + kb_ + woff_, (lds_void *)sa_, 16, 0, 0);               \
         } else {                                                                                             \
-            __builtin_amdgcn_global_load_lds(hbytes + kb_ + hoff[(j_) >> 1], (lds_void *)(sa_ + LM_BM * LM_BK), 16, 0, 0); \
+            __builtin_amdgcn_global_load_lds(hbytes + kb_ + hoff[(c_) >> 1], (lds_void *)(sa_ + LM_BM * LM_BK), 16, 0, 0); \
         }                                                                                                    \
     } while (0)
 
     // Copy cursor: the next slab to request.  Past the last slab of this workgroup it stays on that slab
-    // (redundant copies into a free stage), so that every step issues the same number of copies and the
-    // vmcnt arithmetic below stays exact.
-    int vt_c = vt_begin, kt_c = 0, stage_c = 0;
+    // (redundant copies into the idle stage), so that every step issues the same copies and has no branch.
+    int vt_c = vt_begin, kt_c = 0;
 #define LM_ADVANCE_COPY_CURSOR()                                      \
     do {                                                              \
         if (kt_c + 1 < nk) ++kt_c;                                    \
         else if (vt_c + 1 < vt_end) { ++vt_c; kt_c = 0; }             \
-        stage_c = stage_c + 1 == LM_STAGES ? 0 : stage_c + 1;         \
     } while (0)
-    // Fragment addresses (bf16 element offsets inside a stage) of this lane: [kk][t] for A and B.
-    int fa_off[2][4], fb_off[2][4];
+    // Fragment addresses (bf16 element offsets inside a stage) of this lane at kk = 0; swz() does not depend
+    // on kk, so the other k-steps are the same address with the chunk XORed.
+    int fa_row[4], fb_row[4], f_swz[4];
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            fa_off[kk][t] = slab_offset(wave_m * 128 + t * 32 + l32, kk * 2 + lhalf);
-            fb_off[kk][t] = LM_BM * LM_BK + slab_offset(wave_n * 128 + t * 32 + l32, kk * 2 + lhalf);
-        }
-#define LM_READ_FRAG(dst_, idx_, stage_)                                                                     \
-    do {                                                                                                     \
-        const uint16_t *st_ = lds + (stage_) * LM_STAGE_ELEMS;                                                \
-        if ((idx_) < 8) dst_##a[(idx_) >> 2][(idx_) & 3] = *reinterpret_cast<const bf16x8 *>(st_ + fa_off[(idx_) >> 2][(idx_) & 3]); \
-        else dst_##b[((idx_) - 8) >> 2][(idx_) & 3] = *reinterpret_cast<const bf16x8 *>(st_ + fb_off[((idx_) - 8) >> 2][(idx_) & 3]); \
-    } while (0)
-
-    // Prologue: request the first LM_STAGES slabs, wait for the first, and read its fragments.
-#pragma unroll
-    for (int pre = 0; pre < LM_STAGES; ++pre) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) LM_ISSUE_ONE(j, vt_c, kt_c, stage_c);
-        LM_ADVANCE_COPY_CURSOR();
+    for (int t = 0; t < 4; ++t) {
+        fa_row[t] = (wave_m * 128 + t * 32 + l32) * LM_BK;
+        fb_row[t] = LM_BM * LM_BK + (wave_n * 128 + t * 32 + l32) * LM_BK;
+        f_swz[t] = swz(t * 32 + l32);  // wave_m * 128 and wave_n * 128 do not change bits 1..3
     }
-    bf16x8 Pa[2][4], Pb[2][4], Qa[2][4], Qb[2][4];  // fragments of the slab in use / of the next slab
-    asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory");  // the first slab has landed
+#define LM_FRAG_A(kk_, t_, st_) (*reinterpret_cast<const bf16x8 *>((st_) + fa_row[t_] + ((((kk_) * 2 + lhalf) ^ f_swz[t_]) << 3)))
+#define LM_FRAG_B(kk_, t_, st_) (*reinterpret_cast<const bf16x8 *>((st_) + fb_row[t_] + ((((kk_) * 2 + lhalf) ^ f_swz[t_]) << 3)))
+
 #pragma unroll
-    for (int i = 0; i < 16; ++i) LM_READ_FRAG(P, i, 0);
+    for (int c = 0; c < 16; ++c) LM_ISSUE_ONE(c, vt_c, kt_c, 0);
+    LM_ADVANCE_COPY_CURSOR();
 
-    // One step: the fragments of slab s are in CUR; while its 32 MFMAs run, the 16 fragment reads of slab
-    // s + 1 go into NXT and the 8 copies of slab s + 4 are requested (into the stage slab s occupied: every
-    // wavefront has its slab-s fragments in registers once it has passed the barrier).  Nothing in the
-    // step waits on LDS or on a copy except the vmcnt / barrier pair at its top.  The order below is pinned
-    // with scheduling barriers: an MFMA blocks the issue port for its 8 passes, so a read that follows its
-    // consumer's predecessors in program order would issue too late to hide its latency.
-#define LM_STEP(CUR, NXT, stage_next_)                                                                       \
-    do {                                                                                                     \
-        /* vmcnt(16): copies are retired in order, slab s + 1 is the oldest of the three in flight;          \
-           lgkmcnt(0): this wavefront's fragment reads of slab s have returned.  A bare s_barrier (no fence:  \
-           a fence would wait for every copy in flight) is enough, the data it orders is covered by the two   \
-           counters. */                                                                                      \
-        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");                           \
-        _Pragma("unroll") for (int g = 0; g < 16; ++g) {                                                     \
-            LM_READ_FRAG(NXT, g, stage_next_);                                                               \
-            if (g < 8) LM_ISSUE_ONE(g, vt_c, kt_c, stage_c);                                                 \
-            _Pragma("unroll") for (int q = 0; q < 2; ++q) {                                                  \
-                const int m_ = g * 2 + q, kk_ = m_ >> 4, tm_ = (m_ >> 2) & 3, tn_ = m_ & 3;                   \
-                acc[tm_][tn_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(CUR##a[kk_][tm_], CUR##b[kk_][tn_], acc[tm_][tn_], 0, 0, 0); \
-            }                                                                                                \
-            __builtin_amdgcn_sched_barrier(0);                                                               \
-        }                                                                                                    \
-        LM_ADVANCE_COPY_CURSOR();                                                                            \
-    } while (0)
-
-    int stage = 0;  // stage of the slab whose fragments are in P
+    int stage = 0;
     for (int vt = vt_begin; vt < vt_end; ++vt) {
         f32x16 acc[4][4];
 #pragma unroll
@@ -201,11 +162,42 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
-        for (int kt = 0; kt < nk; kt += 2) {  // nk is even (hidden_dim % 64 == 0)
-            const int s1 = (stage + 1) & (LM_STAGES - 1), s2 = (stage + 2) & (LM_STAGES - 1);
-            LM_STEP(P, Q, s1);
-            LM_STEP(Q, P, s2);
-            stage = s2;
+        for (int kt = 0; kt < nk; ++kt) {
+            // vmcnt(0): this wavefront's copies of slab (vt, kt), requested one step ago, have landed;
+            // lgkmcnt(0): its fragment reads of the previous slab have returned.  After the barrier the
+            // whole slab is in LDS and the other stage is free.  A bare s_barrier is enough (the data it
+            // orders is covered by the two counters).
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            const uint16_t *st = lds + stage * LM_STAGE_ELEMS;
+            bf16x8 fa[2][4], fb[2][4];
+            // Pinned instruction order (an MFMA blocks the issue port for its 8 passes, so a read that follows
+            // its consumer's predecessors in program order would issue too late to hide its latency):
+            // the 8 fragment reads of k-step 0; then every k-step is 8 pairs of MFMAs, the first 4 pairs each
+            // preceded by two fragment reads of the next k-step, and the first 16 pairs of the slab by one
+            // copy of the next slab each.
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                fa[0][t] = LM_FRAG_A(0, t, st);
+                fb[0][t] = LM_FRAG_B(0, t, st);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < 32; ++g) {
+                const int kk = g >> 3, sub = g & 7;  // 8 groups of 2 MFMAs per k-step
+                if (kk < 3 && sub < 4) {  // both reads early in the k-step: they have returned when it ends
+                    fa[(kk + 1) & 1][sub] = LM_FRAG_A(kk + 1, sub, st);
+                    fb[(kk + 1) & 1][sub] = LM_FRAG_B(kk + 1, sub, st);
+                }
+                if (g < 16) LM_ISSUE_ONE(g, vt_c, kt_c, stage ^ 1);
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int m = sub * 2 + q, tm = m >> 2, tn = m & 3;
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][tm], fb[kk & 1][tn], acc[tm][tn], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            LM_ADVANCE_COPY_CURSOR();
+            stage ^= 1;
         }
 
         // ---- the logits of this vocabulary tile are complete: fold them into the running state ----
@@ -346,8 +338,8 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     if (hidden == nullptr || weight == nullptr || ids == nullptr || out == nullptr)
         return fail(KA_ERR_BAD_ARG, "lmhead: null hidden / weight / ids / out pointer");
     if (hidden_dim < 8 || vocab < 1) return fail(KA_ERR_BAD_ARG, "lmhead: hidden_dim %lld, vocab %lld", (long long)hidden_dim, (long long)vocab);
-    if (hidden_dim % (2 * LM_BK) != 0)
-        return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden_dim %lld is not a multiple of %d", (long long)hidden_dim, 2 * LM_BK);
+    if (hidden_dim % LM_BK != 0)
+        return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden_dim %lld is not a multiple of %d", (long long)hidden_dim, LM_BK);
     if (reinterpret_cast<uintptr_t>(hidden) % 16 != 0 || reinterpret_cast<uintptr_t>(weight) % 16 != 0)
         return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden and weight must be 16-byte aligned");
     if (n_rows >= (int64_t(1) << 31) || vocab >= (int64_t(1) << 31) || hidden_dim >= (int64_t(1) << 31))
