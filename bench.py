@@ -92,6 +92,33 @@ def sampling_latency(sampler, steps: int, warmup: int):
     return out
 
 
+def backward_throughput(sampler, iters: int = 5):
+    """Backward of the logprob operator, in place, on bf16 logits [64, 512, 128256] (seed 0)."""
+    import torch
+    from benchmarks.workloads import spike_logits
+
+    n = 64 * 512
+    logits, ids = spike_logits(n, V, seed=0, device="cuda")
+    grad = torch.ones(n, device="cuda")
+    logp = sampler.compute_logp(logits, ids)
+    work = logits.clone()
+    for _ in range(2):
+        sampler.compute_logp_backward(work, ids, logp, grad, inplace=True)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(iters):  # the values degrade from pass to pass, the traffic does not
+        sampler.compute_logp_backward(work, ids, logp, grad, inplace=True)
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / iters
+    gbps = n * (4 * V + 16) / (ms * 1e-3) / 1e9
+    return {"config": "bf16 logits [64,512,128256], gradient written in place; 4*V + 16 bytes per token",
+            "ms": ms, "tokens_per_s": n / (ms * 1e-3),
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel": "logprob_backward_rows<Bf16,256,4,vec>"}}
+
+
 def lmhead_throughput(sampler, iters: int = 3):
     """Fused lm_head -> logprob on hidden bf16 [32768, 4096] x W bf16 [128256, 4096] (seed 0)."""
     import torch
@@ -218,6 +245,7 @@ def main() -> int:
         result["cpu_baseline"] = cpu_baseline(logits, ids, args.cpu_sample_rows)
     del logits3, ids2, logits, ids
     torch.cuda.empty_cache()
+    result["logprob_backward"] = backward_throughput(sampler)
     result["sampling"] = sampling_latency(sampler, args.steps, args.warmup)
     if not args.skip_lmhead:
         result["fused_lm_head"] = lmhead_throughput(sampler)

@@ -73,6 +73,27 @@ int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_t vocab, i
                             const int64_t *ids, float *out, float *entropy, void *hip_stream);
 
 /*
+ * Backward of ka_logprob_*:
+ *     dlogits[r, v] = grad[r] * ((v == ids[r]) - softmax(logits[r, :])[v])
+ * in the logits' dtype.  logp is the forward result for the same (logits, ids);
+ * the row's log-sum-exp is recovered from it, so each logit is read once and
+ * its gradient written once.  dlogits may be the logits buffer itself (same
+ * stride): the gradient then overwrites the logits and no second tensor of
+ * their size exists.  No counterpart in the reference, whose operators run under
+ * torch.inference_mode() (rl_engine/kernels/sampling.py:38,91); this is the
+ * gradient autograd would build for sampling.py:108-110.
+ */
+int ka_logprob_backward_bf16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                             const int64_t *ids, const float *logp, const float *grad, void *dlogits,
+                             int64_t dlogits_stride, void *hip_stream);
+int ka_logprob_backward_f16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                            const int64_t *ids, const float *logp, const float *grad, void *dlogits,
+                            int64_t dlogits_stride, void *hip_stream);
+int ka_logprob_backward_f32(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                            const int64_t *ids, const float *logp, const float *grad, void *dlogits,
+                            int64_t dlogits_stride, void *hip_stream);
+
+/*
  * Fused temperature -> top-k -> top-p -> draw, one token id per row.
  * Replaces SamplerBackend.sample (rl_engine/kernels/sampling.py:39-88) with the
  * filter semantics of native_sampling (benchmarks/benchmark_sampling.py:12-37):

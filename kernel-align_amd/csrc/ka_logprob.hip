@@ -206,3 +206,175 @@ KA_EXPORT int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_
                                       float *entropy, void *hip_stream) {
     return ka::launch<ka::Bf16, true>(logits, n_rows, vocab, row_stride, ids, out, entropy, hip_stream);
 }
+
+// ---------------------------------------------------------------------------
+// Backward of the per-token logprob:
+//     dlogits[r, v] = grad[r] * ((v == ids[r]) - softmax(logits[r, :])[v])
+// One pass: the row's log-sum-exp is recovered from the forward result
+// (lse = logits[r, ids[r]] - logp[r]), every logit is read once and its
+// gradient written once, in the logits' dtype.  dlogits may alias logits (each
+// element is read and then written by the same lane), so the gradient of a
+// [G, L, V] tensor needs no second tensor of that size.
+// ---------------------------------------------------------------------------
+namespace ka {
+namespace {
+
+template <typename T> struct Narrow;
+template <> struct Narrow<Bf16> {
+    static __device__ __forceinline__ uint16_t one(float v) {
+        union { __bf16 b; uint16_t u; } c;
+        c.b = (__bf16)v;  // round to nearest even
+        return c.u;
+    }
+};
+template <> struct Narrow<F16> {
+    static __device__ __forceinline__ uint16_t one(float v) {
+        union { _Float16 h; uint16_t u; } c;
+        c.h = (_Float16)v;
+        return c.u;
+    }
+};
+template <> struct Narrow<F32> {
+    static __device__ __forceinline__ uint32_t one(float v) { return __float_as_uint(v); }
+};
+
+template <typename T> __device__ __forceinline__ uint4 pack_vec(const float (&g)[8]);
+template <typename T> __device__ __forceinline__ uint4 pack_vec(const float (&g)[4]);
+template <> __device__ __forceinline__ uint4 pack_vec<Bf16>(const float (&g)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = uint32_t(Narrow<Bf16>::one(g[2 * j])) | (uint32_t(Narrow<Bf16>::one(g[2 * j + 1])) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+template <> __device__ __forceinline__ uint4 pack_vec<F16>(const float (&g)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = uint32_t(Narrow<F16>::one(g[2 * j])) | (uint32_t(Narrow<F16>::one(g[2 * j + 1])) << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+template <> __device__ __forceinline__ uint4 pack_vec<F32>(const float (&g)[4]) {
+    return make_uint4(__float_as_uint(g[0]), __float_as_uint(g[1]), __float_as_uint(g[2]), __float_as_uint(g[3]));
+}
+
+static __device__ __forceinline__ void store_stream(uint4 *p, const uint4 &v) {
+    u32x4 q = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(q, reinterpret_cast<u32x4 *>(p));
+}
+
+template <typename T, int THREADS, int UNROLL, bool VEC>
+__global__ __launch_bounds__(THREADS) void logprob_backward_rows(const typename T::raw_t *logits,
+                                                                 int64_t n_rows, int vocab, int64_t row_stride,
+                                                                 const int64_t *__restrict__ ids,
+                                                                 const float *__restrict__ logp,
+                                                                 const float *__restrict__ grad,
+                                                                 typename T::raw_t *dlogits, int64_t d_stride) {
+    constexpr int EPV = T::kPerVec;
+    __shared__ float s_lse;
+    const int tid = threadIdx.x;
+    for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+        const typename T::raw_t *rp = logits + row * row_stride;
+        typename T::raw_t *dp = dlogits + row * d_stride;
+        const int64_t id = ids[row];
+        const bool id_ok = id >= 0 && id < vocab;
+        const float g = grad[row];
+        // lse = x_t - logp; an id outside the vocabulary has no defined forward value: its row gets NaN.
+        // One lane reads x_t and the barrier comes before any store, because dlogits may be the logits.
+        if (tid == 0) s_lse = id_ok ? T::widen(rp[id]) - logp[row] : __builtin_nanf("");
+        __syncthreads();
+        const float lse = s_lse;
+        const float nl2 = -lse * kLog2e;
+        const float ng = -g;
+        // d = g * (onehot - p) = -g * p (+ g at the target)
+        auto grad_of = [&](float x, int idx) {
+            const float p = fast_exp2(fmaf(x, kLog2e, nl2));
+            float d = ng * p;
+            if (idx == int(id)) d += g;
+            return d;
+        };
+        if (VEC) {
+            const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+            uint4 *op = reinterpret_cast<uint4 *>(dp);
+            const int nvec = vocab / EPV;
+            int i = tid;
+            for (; i + (UNROLL - 1) * THREADS < nvec; i += UNROLL * THREADS) {
+                uint4 v[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) v[u] = load_stream(vp + i + u * THREADS);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    float x[EPV], d[EPV];
+                    T::unpack(v[u], x);
+#pragma unroll
+                    for (int j = 0; j < EPV; ++j) d[j] = grad_of(x[j], (i + u * THREADS) * EPV + j);
+                    store_stream(op + i + u * THREADS, pack_vec<T>(d));
+                }
+            }
+            for (; i < nvec; i += THREADS) {
+                float x[EPV], d[EPV];
+                T::unpack(load_stream(vp + i), x);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) d[j] = grad_of(x[j], i * EPV + j);
+                store_stream(op + i, pack_vec<T>(d));
+            }
+            const int t = nvec * EPV + tid;
+            if (t < vocab) dp[t] = Narrow<T>::one(grad_of(T::widen(rp[t]), t));
+        } else {
+            for (int i = tid; i < vocab; i += THREADS) dp[i] = Narrow<T>::one(grad_of(T::widen(rp[i]), i));
+        }
+        __syncthreads();  // s_lse is rewritten for the next row
+    }
+}
+
+template <typename T>
+int launch_backward(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride, const int64_t *ids,
+                    const float *logp, const float *grad, void *dlogits, int64_t d_stride, void *hip_stream) {
+    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "logprob backward: n_rows %lld < 0", (long long)n_rows);
+    if (n_rows == 0) return KA_OK;
+    if (logits == nullptr || ids == nullptr || logp == nullptr || grad == nullptr || dlogits == nullptr)
+        return fail(KA_ERR_BAD_ARG, "logprob backward: null pointer argument");
+    if (vocab < 1) return fail(KA_ERR_BAD_ARG, "logprob backward: vocab %lld < 1", (long long)vocab);
+    if (vocab >= (int64_t(1) << 31))
+        return fail(KA_ERR_UNSUPPORTED, "logprob backward: vocab %lld does not fit 31 bits", (long long)vocab);
+    if (row_stride < vocab || d_stride < vocab)
+        return fail(KA_ERR_BAD_ARG, "logprob backward: a row stride is smaller than vocab %lld", (long long)vocab);
+    if (dlogits == logits && d_stride != row_stride)
+        return fail(KA_ERR_BAD_ARG, "logprob backward: in-place use needs equal strides");
+    constexpr int THREADS = 256;
+    constexpr int UNROLL = 4;
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const auto *lp = static_cast<const typename T::raw_t *>(logits);
+    auto *dp = static_cast<typename T::raw_t *>(dlogits);
+    const bool aligned = reinterpret_cast<uintptr_t>(logits) % 16 == 0 && reinterpret_cast<uintptr_t>(dlogits) % 16 == 0 &&
+                         (row_stride * T::kBytes) % 16 == 0 && (d_stride * T::kBytes) % 16 == 0;
+    const unsigned grid = unsigned(n_rows < (int64_t(1) << 30) ? n_rows : (int64_t(1) << 30));
+    if (aligned) {
+        hipLaunchKernelGGL((logprob_backward_rows<T, THREADS, UNROLL, true>), dim3(grid), dim3(THREADS), 0, stream, lp,
+                           n_rows, int(vocab), row_stride, ids, logp, grad, dp, d_stride);
+    } else {
+        hipLaunchKernelGGL((logprob_backward_rows<T, THREADS, 1, false>), dim3(grid), dim3(THREADS), 0, stream, lp,
+                           n_rows, int(vocab), row_stride, ids, logp, grad, dp, d_stride);
+    }
+    return check_hip(hipGetLastError(), "logprob backward launch");
+}
+
+}  // namespace
+}  // namespace ka
+
+KA_EXPORT int ka_logprob_backward_bf16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                       const int64_t *ids, const float *logp, const float *grad, void *dlogits,
+                                       int64_t dlogits_stride, void *hip_stream) {
+    return ka::launch_backward<ka::Bf16>(logits, n_rows, vocab, row_stride, ids, logp, grad, dlogits, dlogits_stride,
+                                         hip_stream);
+}
+KA_EXPORT int ka_logprob_backward_f16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                      const int64_t *ids, const float *logp, const float *grad, void *dlogits,
+                                      int64_t dlogits_stride, void *hip_stream) {
+    return ka::launch_backward<ka::F16>(logits, n_rows, vocab, row_stride, ids, logp, grad, dlogits, dlogits_stride,
+                                        hip_stream);
+}
+KA_EXPORT int ka_logprob_backward_f32(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                      const int64_t *ids, const float *logp, const float *grad, void *dlogits,
+                                      int64_t dlogits_stride, void *hip_stream) {
+    return ka::launch_backward<ka::F32>(logits, n_rows, vocab, row_stride, ids, logp, grad, dlogits, dlogits_stride,
+                                        hip_stream);
+}

@@ -23,6 +23,8 @@ DEFAULT_CHUNK_TOKENS = 8192
 
 _LOGPROB_FN = {torch.bfloat16: "ka_logprob_bf16", torch.float16: "ka_logprob_f16",
                torch.float32: "ka_logprob_f32"}
+_BACKWARD_FN = {torch.bfloat16: "ka_logprob_backward_bf16", torch.float16: "ka_logprob_backward_f16",
+                torch.float32: "ka_logprob_backward_f32"}
 _SAMPLE_FN = {torch.bfloat16: "ka_sample_topk_topp_bf16", torch.float16: "ka_sample_topk_topp_f16",
               torch.float32: "ka_sample_topk_topp_f32"}
 
@@ -125,6 +127,45 @@ class SamplerBackend(nn.Module):
                 _hip.check(status, "ka_logprob_entropy_bf16")
         shape = tuple(logits.shape[:-1])
         return out.view(shape), ent.view(shape)
+
+    @torch.inference_mode()
+    def compute_logp_backward(self, logits, token_ids, logp, grad_logp, inplace=False, chunk_tokens=None):
+        """Gradient of ``compute_logp`` with respect to the logits, in the logits' dtype.
+
+        ``dlogits[..., v] = grad_logp[...] * ((v == token_id) - softmax(logits)[..., v])``.  ``logp`` is the
+        fp32 result of ``compute_logp(logits, token_ids)``; the kernel recovers each row's log-sum-exp from
+        it and touches every logit once.  With ``inplace=True`` the gradient overwrites ``logits`` (which
+        must be row-contiguous) and no second [G, L, V] tensor is allocated.
+        """
+        _require_gpu(logits, "logits")
+        fn_name = _BACKWARD_FN.get(logits.dtype)
+        if fn_name is None:
+            raise TypeError(f"unsupported logits dtype {logits.dtype}")
+        lead = tuple(logits.shape[:-1])
+        if tuple(token_ids.shape) != lead or tuple(logp.shape) != lead or tuple(grad_logp.shape) != lead:
+            raise ValueError("token_ids, logp and grad_logp must have shape logits.shape[:-1]")
+        rows = _rows_view(logits)
+        n_rows, vocab = rows.shape
+        if inplace and rows.data_ptr() != logits.data_ptr():
+            raise ValueError("inplace=True needs row-contiguous logits")
+        ids = token_ids.to(device=logits.device, dtype=torch.int64).contiguous().view(-1)
+        lp = logp.to(device=logits.device, dtype=torch.float32).contiguous().view(-1)
+        g = grad_logp.to(device=logits.device, dtype=torch.float32).contiguous().view(-1)
+        out_rows = rows if inplace else torch.empty((n_rows, vocab), dtype=logits.dtype, device=logits.device)
+        row_stride = rows.stride(0) if n_rows > 1 else vocab
+        out_stride = out_rows.stride(0) if n_rows > 1 else vocab
+        esize = rows.element_size()
+        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
+        fn = getattr(self._lib, fn_name)
+        with torch.cuda.device(logits.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            for start in range(0, n_rows, chunk):
+                n = min(chunk, n_rows - start)
+                status = fn(rows.data_ptr() + start * row_stride * esize, n, vocab, row_stride,
+                            ids.data_ptr() + start * 8, lp.data_ptr() + start * 4, g.data_ptr() + start * 4,
+                            out_rows.data_ptr() + start * out_stride * esize, out_stride, stream)
+                _hip.check(status, fn_name)
+        return logits if inplace else out_rows.view(logits.shape)
 
     # ----------------------------------------------------------------- sampling
     @torch.inference_mode()

@@ -93,3 +93,21 @@ def lmhead_logprob_ref(hidden: torch.Tensor, weight: torch.Tensor, token_ids: to
         lse = m.squeeze(-1) + torch.log(torch.exp(logits - m).sum(dim=-1))
         out[s:s + chunk_rows] = logits.gather(-1, ids[s:s + chunk_rows].unsqueeze(-1)).squeeze(-1) - lse
     return out.view(tuple(hidden.shape[:-1]))
+
+
+def logprob_backward_ref(logits: torch.Tensor, token_ids: torch.Tensor, grad_logp: torch.Tensor,
+                         dtype=torch.float32) -> torch.Tensor:
+    """Gradient of logprob_ref with respect to the logits, by torch autograd on the CPU (in `dtype`):
+    what autograd builds for rl_engine/kernels/sampling.py:108-110 when it is not under inference_mode."""
+    x = logits.detach().cpu().to(dtype).clone().requires_grad_(True)
+    lp = torch.log_softmax(x, dim=-1).gather(-1, token_ids.cpu().to(torch.int64).unsqueeze(-1)).squeeze(-1)
+    lp.backward(grad_logp.detach().cpu().to(dtype))
+    return x.grad
+
+
+def logprob_backward_closed_form(logits: torch.Tensor, token_ids: torch.Tensor, grad_logp: torch.Tensor) -> torch.Tensor:
+    """The same gradient written out in fp64: g * (onehot - softmax)."""
+    x = logits.detach().cpu().double()
+    p = torch.softmax(x, dim=-1)
+    onehot = torch.zeros_like(p).scatter_(-1, token_ids.cpu().to(torch.int64).unsqueeze(-1), 1.0)
+    return grad_logp.detach().cpu().double().unsqueeze(-1) * (onehot - p)

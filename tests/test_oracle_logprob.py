@@ -95,3 +95,25 @@ def test_entropy_closed_forms():
     x = torch.full((1, v), -math.inf, dtype=torch.bfloat16)
     x[0, 3] = 1.0
     assert O.entropy_f64(x).item() == 0.0
+
+
+def test_backward_closed_form_is_autograd():
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(16, 999, generator=g) * 3
+    ids = torch.randint(0, 999, (16,), generator=g)
+    grad = torch.randn(16, generator=g)
+    a = O.logprob_backward_ref(logits, ids, grad, dtype=torch.float64)
+    b = O.logprob_backward_closed_form(logits, ids, grad)
+    assert (a - b).abs().max().item() < 1e-14
+    assert (a.sum(-1)).abs().max().item() < 1e-13          # rows of the gradient sum to zero
+    # finite differences of the fp64 forward pin the sign and the one-hot term
+    x = logits[:2, :50].double()
+    i2, g2 = ids[:2] % 50, grad[:2].double()
+    base = (O.logprob_f64(x, i2) * g2).sum()
+    eps = 1e-6
+    an = O.logprob_backward_closed_form(x, i2, g2)
+    for (r, c) in ((0, int(i2[0])), (0, 3), (1, 17)):
+        xp = x.clone()
+        xp[r, c] += eps
+        fd = ((O.logprob_f64(xp, i2) * g2).sum() - base) / eps
+        assert abs(fd.item() - an[r, c].item()) < 1e-5
