@@ -124,6 +124,21 @@ int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, in
                             void *hip_stream);
 
 /*
+ * The same operator with per-row parameters and the sampled entry's log-probability.
+ * dtype is a KA_DTYPE_* code.  Each of temperature_rows / top_k_rows / top_p_rows is either null (the
+ * scalar next to it applies to every row) or a device array of `batch` values that replaces the scalar; a
+ * row value that is not valid switches that filter off for the row (temperature <= 0 or NaN -> 1,
+ * top_k < 0 -> off, top_p outside (0, 1] -> off).  out_logprob (optional, fp32 [batch]) receives
+ * log(mass of the sampled entry / total surviving mass), the log-probability under the distribution the
+ * entry was drawn from.  The reference takes scalars only (rl_engine/kernels/sampling.py:39); the
+ * FlashInfer operators it forwards to accept per-row tensors (sampling.py:62-64).
+ */
+int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                 float temperature, const float *temperature_rows, int32_t top_k, const int32_t *top_k_rows,
+                 float top_p, const float *top_p_rows, const float *uniforms, int64_t *out_ids,
+                 float *out_logprob, void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/*
  * Fused lm_head -> logprob without materialised logits:
  *     out[r] = h_r . W[ids[r]] - logsumexp_v(h_r . W[v])               (fp32)
  * hidden: bf16 [n_rows, hidden_dim] row-major; weight: bf16 [vocab, hidden_dim]

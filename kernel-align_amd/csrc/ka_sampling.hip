@@ -68,6 +68,11 @@ __device__ __forceinline__ uint64_t weight_fix(float d) {
     return (uint64_t)__dmul_rn(p, scale);
 }
 
+// log(w / z) for integer masses, in fp64 (w >= 1: an entry of mass 0 is never drawn).
+__device__ __forceinline__ float log_ratio(uint64_t w, uint64_t z) {
+    return float(log(double(w)) - log(double(z)));
+}
+
 // floor(s * z) for an fp32 0 <= s < 1 and z < 2^62.
 __device__ __forceinline__ uint64_t floor_scale(float s, uint64_t z) {
     const uint32_t b = __float_as_uint(s);
@@ -308,7 +313,7 @@ template <typename T> __device__ __forceinline__ uint32_t key_step() {
 template <typename T>
 __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *rp, int vocab, bool vec, float temp,
                                           bool has_t, int top_k, bool use_p, float top_p, float u,
-                                          int64_t *out_slot) {
+                                          int64_t *out_slot, float *lp_slot) {
     const int tid = threadIdx.x;
     // 1. lane maxima of the raw values (float max: one convert and half a v_max3 per element; which of
     //    -0 / +0 it returns does not matter, any lower bound of the top_k-th element will do)
@@ -492,24 +497,47 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     }
     __syncthreads();
     if (tid == 0) *out_slot = sh.hit;
+    if (lp_slot != nullptr && tid < int(nb) && int64_t(sh.c.sidx[tid]) == sh.hit) *lp_slot = log_ratio(sh.c.w[tid], z_kept);
     return true;
 }
+
+// Per-launch parameters.  Each of the three filter parameters is either one value for the whole batch or,
+// when its *_rows pointer is set, one value per row; a row value that is not valid switches that filter
+// off (temperature <= 0 or NaN -> 1, top_k < 0 -> off, top_p outside (0, 1] -> off).
+struct SampleParams {
+    float temperature;
+    int top_k;
+    float top_p;
+    const float *temperature_rows;
+    const int32_t *top_k_rows;
+    const float *top_p_rows;
+    const float *uniforms;
+    int64_t *out_ids;
+    float *out_logprob;  // optional: log of the sampled entry's probability under the filtered distribution
+};
 
 // ---------------------------------------------------------------------------
 // The kernel
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t *__restrict__ logits,
-                                                         int vocab, int64_t row_stride, float temp,
-                                                         int top_k, float top_p,
-                                                         const float *__restrict__ uniforms,
-                                                         int64_t *__restrict__ out, int vec, int no_fast) {
+                                                         int vocab, int64_t row_stride, SampleParams prm, int vec,
+                                                         int no_fast) {
     constexpr int EPV = T::kPerVec;
     constexpr int LEVELS = Round<T>::kLevels;
     __shared__ Shared sh;
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.x;
     const typename T::raw_t *rp = logits + row * row_stride;
+    float temp = prm.temperature;
+    int top_k = prm.top_k;
+    float top_p = prm.top_p;
+    if (prm.temperature_rows != nullptr) { temp = prm.temperature_rows[row]; if (!(temp > 0.0f)) temp = 1.0f; }
+    if (prm.top_k_rows != nullptr) { top_k = prm.top_k_rows[row]; if (top_k < 0) top_k = 0; }
+    if (prm.top_p_rows != nullptr) { top_p = prm.top_p_rows[row]; if (!(top_p > 0.0f && top_p <= 1.0f)) top_p = 1.0f; }
+    const float *__restrict__ uniforms = prm.uniforms;
+    int64_t *__restrict__ out = prm.out_ids;
+    float *lp_slot = prm.out_logprob != nullptr ? prm.out_logprob + row : nullptr;
     const bool has_t = temp != 1.0f;
     const bool use_k = top_k > 0 && top_k < vocab;
     const bool use_p = top_p < 1.0f;
@@ -519,7 +547,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (u >= 1.0f) u = __uint_as_float(0x3f7fffffu);
 
     if (use_k && top_k <= S_THREADS && !no_fast) {
-        if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row)) return;
+        if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot)) return;
         __syncthreads();
     }
 
@@ -691,14 +719,17 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
 #pragma unroll
             for (int j = 0; j < EPV; ++j) {
                 cum += w[j];
-                if (cum > tau) { sh.hit = base + j; break; }
+                if (cum > tau) { sh.hit = base + j; sh.pick_z = w[j]; break; }
             }
         }
         carry_mass += tot;
         if (carry_mass > tau) break;  // block-uniform: the hit lies in this tile
     }
     __syncthreads();
-    if (tid == 0) out[row] = sh.hit;
+    if (tid == 0) {
+        out[row] = sh.hit;
+        if (lp_slot != nullptr) *lp_slot = sh.hit >= 0 ? log_ratio(sh.pick_z, z_kept) : __builtin_nanf("");
+    }
 }
 
 // KA_SAMPLE_RADIX_ONLY=1 switches the top-k fast path off (the tests use it to run both paths on every case).
@@ -708,21 +739,22 @@ inline bool force_radix_path() {
 }
 
 template <typename T>
-int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride, float temperature,
-           int32_t top_k, float top_p, const float *uniforms, int64_t *out_ids, void *workspace,
-           size_t workspace_bytes, void *hip_stream) {
+int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride, const SampleParams &prm,
+           void *workspace, size_t workspace_bytes, void *hip_stream) {
     if (batch < 0) return fail(KA_ERR_BAD_ARG, "sample: batch %lld < 0", (long long)batch);
     if (batch == 0) return KA_OK;
-    if (logits == nullptr || uniforms == nullptr || out_ids == nullptr)
+    if (logits == nullptr || prm.uniforms == nullptr || prm.out_ids == nullptr)
         return fail(KA_ERR_BAD_ARG, "sample: null logits / uniforms / out_ids pointer");
     if (vocab < 1) return fail(KA_ERR_BAD_ARG, "sample: vocab %lld < 1", (long long)vocab);
     if (vocab >= (int64_t(1) << 22))
         return fail(KA_ERR_UNSUPPORTED, "sample: vocab %lld >= 2^22 (integer masses would overflow)",
                     (long long)vocab);
     if (row_stride < vocab) return fail(KA_ERR_BAD_ARG, "sample: row_stride < vocab");
-    if (!(temperature > 0.0f)) return fail(KA_ERR_BAD_ARG, "sample: temperature %g must be > 0", temperature);
-    if (top_k < 0) return fail(KA_ERR_BAD_ARG, "sample: top_k %d < 0", top_k);
-    if (!(top_p > 0.0f && top_p <= 1.0f)) return fail(KA_ERR_BAD_ARG, "sample: top_p %g outside (0, 1]", top_p);
+    if (prm.temperature_rows == nullptr && !(prm.temperature > 0.0f))
+        return fail(KA_ERR_BAD_ARG, "sample: temperature %g must be > 0", prm.temperature);
+    if (prm.top_k_rows == nullptr && prm.top_k < 0) return fail(KA_ERR_BAD_ARG, "sample: top_k %d < 0", prm.top_k);
+    if (prm.top_p_rows == nullptr && !(prm.top_p > 0.0f && prm.top_p <= 1.0f))
+        return fail(KA_ERR_BAD_ARG, "sample: top_p %g outside (0, 1]", prm.top_p);
     if (batch >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "sample: batch too large");
     if (workspace_bytes < ka_sample_workspace_bytes(batch, vocab) || (workspace == nullptr && workspace_bytes > 0))
         return fail(KA_ERR_WORKSPACE, "sample: workspace of %zu B, need %zu B", workspace_bytes,
@@ -730,9 +762,30 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
     const bool aligned = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * T::kBytes) % 16 == 0);
     hipLaunchKernelGGL((sample_rows<T>), dim3(unsigned(batch)), dim3(S_THREADS), 0,
                        static_cast<hipStream_t>(hip_stream),
-                       static_cast<const typename T::raw_t *>(logits), int(vocab), row_stride, temperature,
-                       int(top_k), top_p, uniforms, out_ids, aligned ? 1 : 0, force_radix_path() ? 1 : 0);
+                       static_cast<const typename T::raw_t *>(logits), int(vocab), row_stride, prm,
+                       aligned ? 1 : 0, force_radix_path() ? 1 : 0);
     return check_hip(hipGetLastError(), "sample launch");
+}
+
+inline SampleParams scalar_params(float temperature, int32_t top_k, float top_p, const float *uniforms,
+                                  int64_t *out_ids) {
+    SampleParams p{};
+    p.temperature = temperature;
+    p.top_k = top_k;
+    p.top_p = top_p;
+    p.uniforms = uniforms;
+    p.out_ids = out_ids;
+    return p;
+}
+
+inline int launch_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                     const SampleParams &prm, void *workspace, size_t workspace_bytes, void *hip_stream) {
+    switch (dtype) {
+        case KA_DTYPE_BF16: return launch<Bf16>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream);
+        case KA_DTYPE_F16: return launch<F16>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream);
+        case KA_DTYPE_F32: return launch<F32>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream);
+        default: return fail(KA_ERR_BAD_ARG, "sample: unknown dtype code %d", dtype);
+    }
 }
 
 }  // namespace
@@ -749,20 +802,36 @@ KA_EXPORT int ka_sample_topk_topp_bf16(const void *logits, int64_t batch, int64_
                                        float temperature, int32_t top_k, float top_p, const float *uniforms,
                                        int64_t *out_ids, void *workspace, size_t workspace_bytes,
                                        void *hip_stream) {
-    return ka::launch<ka::Bf16>(logits, batch, vocab, row_stride, temperature, top_k, top_p, uniforms, out_ids,
-                                workspace, workspace_bytes, hip_stream);
+    return ka::launch<ka::Bf16>(logits, batch, vocab, row_stride,
+                              ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids), workspace,
+                              workspace_bytes, hip_stream);
 }
 KA_EXPORT int ka_sample_topk_topp_f16(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                                       float temperature, int32_t top_k, float top_p, const float *uniforms,
                                       int64_t *out_ids, void *workspace, size_t workspace_bytes,
                                       void *hip_stream) {
-    return ka::launch<ka::F16>(logits, batch, vocab, row_stride, temperature, top_k, top_p, uniforms, out_ids,
-                               workspace, workspace_bytes, hip_stream);
+    return ka::launch<ka::F16>(logits, batch, vocab, row_stride,
+                              ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids), workspace,
+                              workspace_bytes, hip_stream);
 }
 KA_EXPORT int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                                       float temperature, int32_t top_k, float top_p, const float *uniforms,
                                       int64_t *out_ids, void *workspace, size_t workspace_bytes,
                                       void *hip_stream) {
-    return ka::launch<ka::F32>(logits, batch, vocab, row_stride, temperature, top_k, top_p, uniforms, out_ids,
-                               workspace, workspace_bytes, hip_stream);
+    return ka::launch<ka::F32>(logits, batch, vocab, row_stride,
+                              ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids), workspace,
+                              workspace_bytes, hip_stream);
+}
+
+KA_EXPORT int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
+                           float temperature, const float *temperature_rows, int32_t top_k,
+                           const int32_t *top_k_rows, float top_p, const float *top_p_rows, const float *uniforms,
+                           int64_t *out_ids, float *out_logprob, void *workspace, size_t workspace_bytes,
+                           void *hip_stream) {
+    ka::SampleParams p = ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids);
+    p.temperature_rows = temperature_rows;
+    p.top_k_rows = top_k_rows;
+    p.top_p_rows = top_p_rows;
+    p.out_logprob = out_logprob;
+    return ka::launch_ex(dtype, logits, batch, vocab, row_stride, p, workspace, workspace_bytes, hip_stream);
 }

@@ -25,6 +25,7 @@ _LOGPROB_FN = {torch.bfloat16: "ka_logprob_bf16", torch.float16: "ka_logprob_f16
                torch.float32: "ka_logprob_f32"}
 _BACKWARD_FN = {torch.bfloat16: "ka_logprob_backward_bf16", torch.float16: "ka_logprob_backward_f16",
                 torch.float32: "ka_logprob_backward_f32"}
+_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 _SAMPLE_FN = {torch.bfloat16: "ka_sample_topk_topp_bf16", torch.float16: "ka_sample_topk_topp_f16",
               torch.float32: "ka_sample_topk_topp_f32"}
 
@@ -170,7 +171,7 @@ class SamplerBackend(nn.Module):
     # ----------------------------------------------------------------- sampling
     @torch.inference_mode()
     def sample(self, logits, top_k=None, top_p=None, temperature=1.0, deterministic=True,
-               uniforms=None, generator=None):
+               uniforms=None, generator=None, return_logprob=False):
         """Draw one token id per row after temperature -> top-k -> top-p filtering.
 
         logits: [B, V] bf16 / fp16 / fp32 on the GPU.  Returns int64 [B] (reference:
@@ -178,44 +179,77 @@ class SamplerBackend(nn.Module):
         ``uniforms`` ([B] fp32 in [0, 1)) drives the draw; if None they come from
         ``torch.rand(B, generator=generator)`` on the logits' device.  The kernels are always
         deterministic, so ``deterministic`` is accepted and ignored.
+
+        ``top_k``, ``top_p`` and ``temperature`` may each be a [B] tensor of per-row values (a row value
+        that is not valid switches that filter off for the row).  With ``return_logprob=True`` the result
+        is ``(ids, logprob)`` where logprob (fp32 [B]) is the log-probability of the drawn token under the
+        filtered, renormalised distribution it was drawn from.
         """
         _require_gpu(logits, "logits")
         if logits.dim() != 2:
             raise ValueError("logits must be [B, V]")
-        fn_name = _SAMPLE_FN.get(logits.dtype)
-        if fn_name is None:
+        if logits.dtype not in _SAMPLE_FN:
             raise TypeError(f"unsupported logits dtype {logits.dtype}")
         batch, vocab = logits.shape
-        k = 0 if top_k is None else int(top_k)
-        if top_k is not None and k < 1:
-            raise ValueError(f"top_k must be >= 1 (got {top_k})")
-        p = 1.0 if top_p is None else float(top_p)
-        if not 0.0 < p <= 1.0:
-            raise ValueError(f"top_p must be in (0, 1] (got {top_p})")
-        temperature = float(temperature)
-        if not temperature > 0.0:
-            raise ValueError(f"temperature must be > 0 (got {temperature})")
+        dev = logits.device
+
+        def rows_or_scalar(value, name, dtype, default, check):
+            if isinstance(value, torch.Tensor):
+                if tuple(value.shape) != (batch,):
+                    raise ValueError(f"{name} tensor must have shape ({batch},)")
+                return default, value.to(device=dev, dtype=dtype).contiguous()
+            scalar = default if value is None else value
+            check(scalar)
+            return scalar, None
+
+        def check_k(v):
+            if top_k is not None and int(v) < 1:
+                raise ValueError(f"top_k must be >= 1 (got {top_k})")
+
+        def check_p(v):
+            if not 0.0 < float(v) <= 1.0:
+                raise ValueError(f"top_p must be in (0, 1] (got {top_p})")
+
+        def check_t(v):
+            if not float(v) > 0.0:
+                raise ValueError(f"temperature must be > 0 (got {temperature})")
+
+        k, k_rows = rows_or_scalar(top_k, "top_k", torch.int32, 0, check_k)
+        p, p_rows = rows_or_scalar(top_p, "top_p", torch.float32, 1.0, check_p)
+        t, t_rows = rows_or_scalar(temperature, "temperature", torch.float32, 1.0, check_t)
+        k, p, t = int(k), float(p), float(t)
         rows = _rows_view(logits)
         if uniforms is None:
-            uniforms = torch.rand(batch, generator=generator, device=logits.device, dtype=torch.float32)
+            uniforms = torch.rand(batch, generator=generator, device=dev, dtype=torch.float32)
         else:
             if tuple(uniforms.shape) != (batch,):
                 raise ValueError(f"uniforms must have shape ({batch},)")
-            uniforms = uniforms.to(device=logits.device, dtype=torch.float32).contiguous()
-        out = torch.empty(batch, dtype=torch.int64, device=logits.device)
+            uniforms = uniforms.to(device=dev, dtype=torch.float32).contiguous()
+        out = torch.empty(batch, dtype=torch.int64, device=dev)
+        logprob = torch.empty(batch, dtype=torch.float32, device=dev) if return_logprob else None
         if batch == 0:
-            return out
+            return (out, logprob) if return_logprob else out
         ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
         self.pool.reset()
-        ws = self.pool.reserve(ws_bytes, logits.device)
+        ws = self.pool.reserve(ws_bytes, dev)
         row_stride = rows.stride(0) if batch > 1 else vocab
-        with torch.cuda.device(logits.device):
+        extended = return_logprob or k_rows is not None or p_rows is not None or t_rows is not None
+        with torch.cuda.device(dev):
             stream = torch.cuda.current_stream().cuda_stream
-            status = getattr(self._lib, fn_name)(
-                rows.data_ptr(), batch, vocab, row_stride, temperature, k, p, uniforms.data_ptr(),
-                out.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+            if extended:
+                fn_name = "ka_sample_ex"
+                ptr = lambda x: None if x is None else x.data_ptr()  # noqa: E731
+                status = self._lib.ka_sample_ex(
+                    _DTYPE_CODE[logits.dtype], rows.data_ptr(), batch, vocab, row_stride, t, ptr(t_rows), k,
+                    ptr(k_rows), p, ptr(p_rows), uniforms.data_ptr(), out.data_ptr(), ptr(logprob),
+                    ws.data_ptr(), ws_bytes, stream)
+            else:
+                fn_name = _SAMPLE_FN[logits.dtype]
+                status = getattr(self._lib, fn_name)(
+                    rows.data_ptr(), batch, vocab, row_stride, t, k, p, uniforms.data_ptr(),
+                    out.data_ptr(), ws.data_ptr(), ws_bytes, stream)
         _hip.check(status, fn_name)
-        return out
+        return (out, logprob) if return_logprob else out
 
     # ---------------------------------------------------------------- fused GEMM
     @torch.inference_mode()

@@ -14,7 +14,7 @@ _DTYPES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
 class RowInfo(ctypes.Structure):
     _fields_ = [("n_topk", c_int64), ("n_kept", c_int64), ("z_topk", c_uint64), ("z_kept", c_uint64),
-                ("kth_value", c_float), ("max_value", c_float)]
+                ("kth_value", c_float), ("max_value", c_float), ("w_pick", c_uint64)]
 
 
 _lib = None
@@ -74,5 +74,39 @@ def sample(logits: torch.Tensor, temperature: float = 1.0, top_k=None, top_p=Non
         raise ValueError(f"ka_oracle_sample rejected its arguments (rc={rc})")
     if return_info:
         return out, [dict(n_topk=i.n_topk, n_kept=i.n_kept, z_topk=i.z_topk, z_kept=i.z_kept,
-                          kth_value=i.kth_value, max_value=i.max_value) for i in info]
+                          kth_value=i.kth_value, max_value=i.max_value, w_pick=i.w_pick) for i in info]
     return out
+
+
+def sample_rows(logits: torch.Tensor, temperature, top_k, top_p, uniforms):
+    """Per-row parameters: each of temperature / top_k / top_p is a scalar, None, or a length-B sequence.
+    A row's invalid value switches that filter off (T <= 0 or NaN -> 1, top_k < 0 -> off, top_p outside
+    (0, 1] -> off), as the kernel does.  Returns (ids int64 [B], logprob float64 [B]) where logprob is the
+    log of the sampled entry's probability under the filtered, renormalised distribution."""
+    import math
+
+    batch = logits.shape[0]
+
+    def per_row(v, default):
+        if v is None:
+            return [default] * batch
+        if isinstance(v, torch.Tensor):
+            v = v.detach().cpu().tolist()
+        if isinstance(v, (list, tuple)):
+            assert len(v) == batch
+            return list(v)
+        return [v] * batch
+
+    ts, ks, ps = per_row(temperature, 1.0), per_row(top_k, 0), per_row(top_p, 1.0)
+    ids = torch.empty(batch, dtype=torch.int64)
+    lps = torch.empty(batch, dtype=torch.float64)
+    for r in range(batch):
+        t = float(torch.tensor(ts[r], dtype=torch.float32))
+        t = t if t > 0.0 else 1.0
+        k = int(ks[r]) if ks[r] is not None and int(ks[r]) > 0 else 0
+        p = float(torch.tensor(1.0 if ps[r] is None else ps[r], dtype=torch.float32))
+        p = p if 0.0 < p <= 1.0 else 1.0
+        out, info = sample(logits[r:r + 1], t, k, p, uniforms[r:r + 1], return_info=True)
+        ids[r] = out[0]
+        lps[r] = math.log(info[0]["w_pick"]) - math.log(info[0]["z_kept"])
+    return ids, lps

@@ -199,6 +199,7 @@ typedef struct {
     uint64_t z_kept;  /* integer mass of B */
     float kth_value;  /* k-th largest scaled logit (or -inf when top-k is off) */
     float max_value;
+    uint64_t w_pick;  /* integer mass of the sampled entry: its probability is w_pick / z_kept */
 } ka_oracle_row_info;
 
 int ka_oracle_sample(const void *logits, int dtype, int64_t batch, int64_t vocab, int64_t row_stride,
@@ -262,9 +263,10 @@ int ka_oracle_sample(const void *logits, int dtype, int64_t batch, int64_t vocab
         uint64_t tau = floor_scale(u, zb);
         uint64_t cum = 0;
         int64_t pick = cand[nb - 1].idx;
+        uint64_t w_pick = w[cand[nb - 1].key];
         for (int64_t j = 0; j < nb; ++j) {
             cum += w[cand[j].key];
-            if (cum > tau) { pick = cand[j].idx; break; }
+            if (cum > tau) { pick = cand[j].idx; w_pick = w[cand[j].key]; break; }
         }
         out_ids[r] = pick;
         if (info) {
@@ -274,6 +276,7 @@ int ka_oracle_sample(const void *logits, int dtype, int64_t batch, int64_t vocab
             info[r].z_kept = zb;
             info[r].kth_value = kth ? bits_to_f32((kth & 0x80000000u) ? (kth & 0x7fffffffu) : ~kth) : -INFINITY;
             info[r].max_value = mx;
+            info[r].w_pick = w_pick;
         }
     }
     free(y); free(keys); free(cand); free(w); free(hist);

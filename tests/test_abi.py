@@ -61,6 +61,12 @@ def test_sampling_argument_checks():
     assert call(p, 2, 128, 128, 1.0, 5, 1.5, p, p, None, 0, None) == _hip.KA_ERR_BAD_ARG
     assert call(p, 2, 1 << 22, 1 << 22, 1.0, 5, 0.9, p, p, None, 0, None) == _hip.KA_ERR_UNSUPPORTED
     assert lib.ka_sample_workspace_bytes(256, 128256) >= 0
+    ex = lib.ka_sample_ex
+    assert ex(0, None, 0, 128, 128, 1.0, None, 0, None, 1.0, None, None, None, None, None, 0, None) == _hip.KA_OK
+    assert ex(7, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 0, None) == _hip.KA_ERR_BAD_ARG   # dtype code
+    assert ex(0, p, 2, 128, 128, 0.0, None, 0, None, 1.0, None, p, p, None, None, 0, None) == _hip.KA_ERR_BAD_ARG   # scalar T
+    # a per-row array replaces its scalar, which is then not checked; no GPU here, so the launch itself fails
+    assert ex(0, p, 2, 128, 128, 0.0, p, -1, p, 9.0, p, p, p, None, None, 0, None) == _hip.KA_ERR_HIP
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

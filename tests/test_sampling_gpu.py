@@ -183,3 +183,39 @@ def test_huge_temperature_folds_values_together(sampler):
     u = torch.rand(8, generator=g)
     for temp in (1e3, 1e30, 3e38):
         check_exact(sampler, logits, u, 50, 0.9, temp)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_per_row_parameters_and_sampled_logprob(sampler, dtype, monkeypatch):
+    g = torch.Generator().manual_seed(41)
+    batch, vocab = 40, 20000
+    logits = (torch.randn(batch, vocab, generator=g) * 3).to(dtype)
+    logits[3] = ((logits[3].float() * 2).round() / 2).to(dtype)          # ties
+    u = torch.rand(batch, generator=g)
+    ks = torch.randint(1, 200, (batch,), generator=g).to(torch.int32)
+    ks[0], ks[1], ks[2] = 0, -5, 5000                                     # off, invalid -> off, radix path
+    ps = (torch.rand(batch, generator=g) * 0.9 + 0.05)
+    ps[4], ps[5] = 1.0, 7.0                                               # off, invalid -> off
+    ts = (torch.rand(batch, generator=g) * 1.5 + 0.3)
+    ts[6], ts[7] = 1.0, -2.0                                              # identity, invalid -> 1
+    want_ids, want_lp = exact.sample_rows(logits, ts, ks, ps, u)
+    for radix_only in (False, True):
+        if radix_only:
+            monkeypatch.setenv("KA_SAMPLE_RADIX_ONLY", "1")
+        ids, lp = sampler.sample(logits.cuda(), top_k=ks.cuda(), top_p=ps.cuda(), temperature=ts.cuda(),
+                                 uniforms=u.cuda(), return_logprob=True)
+        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
+        assert torch.equal(ids.cpu(), want_ids)
+        assert (lp.cpu().double() - want_lp).abs().max().item() < 1e-5
+        assert (lp <= 0).all()
+    # scalar parameters through the extended entry point give the scalar entry point's ids
+    ids2, lp2 = sampler.sample(logits.cuda(), top_k=50, top_p=0.9, temperature=0.7, uniforms=u.cuda(), return_logprob=True)
+    assert torch.equal(ids2, sampler.sample(logits.cuda(), top_k=50, top_p=0.9, temperature=0.7, uniforms=u.cuda()))
+    w_ids, w_lp = exact.sample_rows(logits, 0.7, 50, 0.9, u)
+    assert torch.equal(ids2.cpu(), w_ids) and (lp2.cpu().double() - w_lp).abs().max().item() < 1e-5
+    # mixing a per-row tensor with scalars
+    ids3 = sampler.sample(logits.cuda(), top_k=ks.cuda(), top_p=0.8, temperature=1.0, uniforms=u.cuda())
+    assert torch.equal(ids3.cpu(), exact.sample_rows(logits, 1.0, ks, 0.8, u)[0])
+    # the log-probability is the one of the filtered distribution: top_k = 1 -> log 1 = 0 without ties
+    _, lp_greedy = sampler.sample(torch.randn(8, 1000, generator=g).cuda(), top_k=1, uniforms=u[:8].cuda(), return_logprob=True)
+    assert (lp_greedy == 0).all()
