@@ -1,0 +1,105 @@
+// Copy side of the fused lm_head kernel in isolation, on the real access pattern: workgroup (token block, split)
+// walks 63 vocabulary tiles x 64 slabs and copies a [256 rows x 128 B] slab of W and one of hidden per step with
+// direct global->LDS copies (rows 8192 B apart, 4 token blocks x 8 splits share an XCD's L2).  Variants:
+//   - copies alone (what the memory system delivers for this pattern, L2 hits and misses included);
+//   - the slab's 64 MFMAs alone (32x32x16 bf16 on registers; no fragment reads, one barrier per slab);
+//   - both, with the copies running LOOK slabs ahead of the one consumed (LOOK = 1 is what two 64 KB stages in
+//     LDS allow: nothing is in flight at the moment a slab is waited for; LDS contents are garbage here, so deeper
+//     lookahead can be timed although it would not fit).
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+typedef __attribute__((address_space(3))) void lds_void;
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template <int LOOK, bool COPY, bool MFMA>
+__global__ __launch_bounds__(256) void k(const char *__restrict__ W, const char *__restrict__ H, int n_splits,
+                                         int tiles_per_split, int nk, unsigned *out) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int total = gridDim.x;
+    const int logical = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;  // consecutive logical ids share an XCD
+    const int tb = logical / n_splits, sp = logical % n_splits;
+    const char *wb = W + size_t(sp) * tiles_per_split * 256 * 8192;
+    const char *hb = H + size_t(tb) * 256 * 8192;
+    const unsigned lane_off = unsigned(wave * 8 + (lane >> 3)) * 8192 + (lane & 7) * 16;
+    const int steps = tiles_per_split * nk;
+    auto issue1 = [&](int s, int c) {
+        if (s >= steps) s = steps - 1;
+        const int vt = s / nk, kt = s % nk;
+        const char *src = ((c & 1) ? hb : wb + size_t(vt) * 256 * 8192) + kt * 128 + lane_off + (c >> 1) * 32 * 8192;
+        unsigned char *dst = lds + (s & 1) * 65536 + wave * 1024 + (c & 1) * 32768 + (c >> 1) * 4096;
+        __builtin_amdgcn_global_load_lds(src, (lds_void *)dst, 16, 0, 0);
+    };
+    if (COPY)
+        for (int s = 0; s < LOOK; ++s)
+#pragma unroll
+            for (int c = 0; c < 16; ++c) issue1(s, c);
+    f32x16 acc[16];
+    for (int i = 0; i < 16; ++i)
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    bf16x8 fa, fb;
+    for (int i = 0; i < 8; ++i) { fa[i] = (__bf16)float(lane + i); fb[i] = (__bf16)float(lane - i); }
+    for (int s = 0; s < steps; ++s) {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(16 * (LOOK - 1)) : "memory");
+#pragma unroll
+        for (int g = 0; g < 32; ++g) {  // one copy per pair of MFMAs in the first half of the slab
+            if (COPY && g < 16) issue1(s + LOOK, g);
+            if (MFMA) {
+                acc[(2 * g) & 15] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[(2 * g) & 15], 0, 0, 0);
+                acc[(2 * g + 1) & 15] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc[(2 * g + 1) & 15], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < 16; ++i)
+        for (int r = 0; r < 16; ++r) t += acc[i][r];
+    if ((lds[threadIdx.x] == 0x7b && steps < 0) || t == 12345.f) out[0] = 1;
+}
+
+int main() {
+    unsigned *o;
+    hipMalloc(&o, 4);
+    const int n_tok_blocks = 128, n_splits = 8, tps = 63, nk = 64;  // hidden [32768, 4096], W [129024, 4096] bf16
+    const size_t wbytes = size_t(n_splits) * tps * 256 * 8192, hbytes = size_t(n_tok_blocks) * 256 * 8192;
+    char *W, *H;
+    hipMalloc(&W, wbytes);
+    hipMalloc(&H, hbytes);
+    hipMemset(W, 1, wbytes);
+    hipMemset(H, 1, hbytes);
+    hipEvent_t e0, e1;
+    hipEventCreate(&e0);
+    hipEventCreate(&e1);
+    const double bytes = double(n_tok_blocks) * n_splits * tps * nk * 65536;
+    const double flops = 2.0 * n_tok_blocks * 256 * double(n_splits) * tps * 256 * 4096;
+    auto run = [&](const char *name, auto kern, bool copies, bool mfma) {
+        hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 131072);
+        float best = 1e9;
+        for (int rep = 0; rep < 3; ++rep) {
+            hipEventRecord(e0);
+            hipLaunchKernelGGL(kern, dim3(n_tok_blocks * n_splits), dim3(256), 131072, 0, W, H, n_splits, tps, nk, o);
+            hipEventRecord(e1);
+            hipEventSynchronize(e1);
+            float ms;
+            hipEventElapsedTime(&ms, e0, e1);
+            if (ms < best) best = ms;
+        }
+        printf("%-44s %7.3f ms", name, best);
+        if (copies) printf("  %6.0f GB/s L2->CU", bytes / best / 1e6);
+        if (mfma) printf("  %5.0f TFLOP/s", flops / best / 1e9);
+        printf("\n");
+        fflush(stdout);
+    };
+    run("copies alone, 1 slab ahead", k<1, true, false>, true, false);
+    run("copies alone, 2 slabs ahead", k<2, true, false>, true, false);
+    run("copies alone, 3 slabs ahead", k<3, true, false>, true, false);
+    run("MFMAs alone (barrier per slab)", k<1, false, true>, false, true);
+    run("copies + MFMAs, 1 slab ahead", k<1, true, true>, true, true);
+    run("copies + MFMAs, 2 slabs ahead", k<2, true, true>, true, true);
+    run("copies + MFMAs, 3 slabs ahead", k<3, true, true>, true, true);
+    return 0;
+}

@@ -148,9 +148,27 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
 #define LM_FRAG_A(kk_, t_, st_) (*reinterpret_cast<const bf16x8 *>((st_) + fa_row[t_] + ((((kk_) * 2 + lhalf) ^ f_swz[t_]) << 3)))
 #define LM_FRAG_B(kk_, t_, st_) (*reinterpret_cast<const bf16x8 *>((st_) + fb_row[t_] + ((((kk_) * 2 + lhalf) ^ f_swz[t_]) << 3)))
 
+    // Software pipeline, per slab s (stage s & 1) in 32 groups of two MFMAs:
+    //   groups  0..7   request copies 8..15 of slab s + 1 (other stage);
+    //   group   24     waits for slab s + 1 (vmcnt(0)) and for this wavefront's last fragment reads of slab s
+    //                  (lgkmcnt(0)), then s_barrier: slab s + 1 is complete in LDS and nobody reads slab s any more;
+    //   groups 24..27  read the k-step-0 fragments of slab s + 1, so that the next slab starts without waiting
+    //                  for LDS;
+    //   groups 24..31  request copies 0..7 of slab s + 2 into the stage slab s has just left.
+    // An MFMA blocks the issue port for its 8 passes, so a read that follows its consumer's predecessors in
+    // program order would issue too late to hide its latency: the order below is pinned with sched_barrier.
 #pragma unroll
     for (int c = 0; c < 16; ++c) LM_ISSUE_ONE(c, vt_c, kt_c, 0);
     LM_ADVANCE_COPY_CURSOR();
+#pragma unroll
+    for (int c = 0; c < 8; ++c) LM_ISSUE_ONE(c, vt_c, kt_c, 1);
+    asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");  // copies complete in order: slab 0 is in
+    bf16x8 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        fa[0][t] = LM_FRAG_A(0, t, lds);
+        fb[0][t] = LM_FRAG_B(0, t, lds);
+    }
 
     int stage = 0;
     for (int vt = vt_begin; vt < vt_end; ++vt) {
@@ -163,40 +181,43 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                 for (int r = 0; r < 16; ++r) acc[tm][tn][r] = 0.0f;
 
         for (int kt = 0; kt < nk; ++kt) {
-            // vmcnt(0): this wavefront's copies of slab (vt, kt), requested one step ago, have landed;
-            // lgkmcnt(0): its fragment reads of the previous slab have returned.  After the barrier the
-            // whole slab is in LDS and the other stage is free.  A bare s_barrier is enough (the data it
-            // orders is covered by the two counters).
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
             const uint16_t *st = lds + stage * LM_STAGE_ELEMS;
-            bf16x8 fa[2][4], fb[2][4];
-            // Pinned instruction order (an MFMA blocks the issue port for its 8 passes, so a read that follows
-            // its consumer's predecessors in program order would issue too late to hide its latency):
-            // the 8 fragment reads of k-step 0; then every k-step is 8 pairs of MFMAs, the first 4 pairs each
-            // preceded by two fragment reads of the next k-step, and the first 16 pairs of the slab by one
-            // copy of the next slab each.
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                fa[0][t] = LM_FRAG_A(0, t, st);
-                fb[0][t] = LM_FRAG_B(0, t, st);
-            }
+            const uint16_t *nst = lds + (stage ^ 1) * LM_STAGE_ELEMS;
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < 32; ++g) {
                 const int kk = g >> 3, sub = g & 7;  // 8 groups of 2 MFMAs per k-step
+                // First MFMA of the pair, then the group's reads and copy (they issue in its shadow), then the
+                // second.  The reads come after an MFMA so that the wait the compiler places in front of the
+                // first MFMA of an iteration does not cover reads issued a moment before.
+                {
+                    const int m = sub * 2, tm = m >> 2, tn = m & 3;
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][tm], fb[kk & 1][tn], acc[tm][tn], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
                 if (kk < 3 && sub < 4) {  // both reads early in the k-step: they have returned when it ends
                     fa[(kk + 1) & 1][sub] = LM_FRAG_A(kk + 1, sub, st);
                     fb[(kk + 1) & 1][sub] = LM_FRAG_B(kk + 1, sub, st);
                 }
-                if (g < 16) LM_ISSUE_ONE(g, vt_c, kt_c, stage ^ 1);
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const int m = sub * 2 + q, tm = m >> 2, tn = m & 3;
+                if (g < 8) LM_ISSUE_ONE(8 + g, vt_c, kt_c, stage ^ 1);
+                if (g == 8) LM_ADVANCE_COPY_CURSOR();
+                if (g == 24) {
+                    // Builtins rather than inline asm: the compiler's own wait-count bookkeeping sees them, so it
+                    // does not add a conservative lgkmcnt(0) behind the fresh reads that follow.
+                    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+                    __builtin_amdgcn_s_barrier();
+                }
+                if (g >= 24 && g < 28) {
+                    fa[0][g - 24] = LM_FRAG_A(0, g - 24, nst);
+                    fb[0][g - 24] = LM_FRAG_B(0, g - 24, nst);
+                }
+                if (g >= 24) LM_ISSUE_ONE(g - 24, vt_c, kt_c, stage);
+                {
+                    const int m = sub * 2 + 1, tm = m >> 2, tn = m & 3;
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][tm], fb[kk & 1][tn], acc[tm][tn], 0, 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            LM_ADVANCE_COPY_CURSOR();
             stage ^= 1;
         }
 
