@@ -233,30 +233,52 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             const bool mine = d >= 0 && d < 128 && ((d >> 2) & 1) == lhalf;
             const int want = mine ? (((d >> 5) << 4) | ((d & 31) >> 3 << 2) | (d & 3)) : -1;  // tm*16 + r
             float mn = m_run[tn];
-#pragma unroll
-            for (int tm = 0; tm < 4; ++tm)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
-                    mn = fmaxf(mn, x);
-                    if (want == tm * 16 + r) xt[tn] = x;
-                }
-            const float ml2n = mn * kLog2e;
             float part[4];
+            // Wavefront-uniform choice: almost every tile lies inside the vocabulary and holds no lane's target,
+            // and then needs neither the bounds select nor the capture compare per logit.
+            if (limit >= 128 && !__any(mine)) {
 #pragma unroll
-            for (int tm = 0; tm < 4; ++tm) {
-                float e[16];
+                for (int tm = 0; tm < 4; ++tm)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
-                    e[r] = fast_exp2(fmaf(x, kLog2e, -ml2n));
+                    for (int r = 0; r < 16; ++r) mn = fmaxf(mn, acc[tm][tn][r]);
+                const float ml2f = mn * kLog2e;
+#pragma unroll
+                for (int tm = 0; tm < 4; ++tm) {
+                    float e[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) e[r] = fast_exp2(fmaf(acc[tm][tn][r], kLog2e, -ml2f));
+#pragma unroll
+                    for (int step = 1; step < 16; step <<= 1)
+#pragma unroll
+                        for (int r = 0; r + step < 16; r += 2 * step) e[r] += e[r + step];
+                    part[tm] = e[0];
                 }
+            } else {
 #pragma unroll
-                for (int step = 1; step < 16; step <<= 1)
+                for (int tm = 0; tm < 4; ++tm)
 #pragma unroll
-                    for (int r = 0; r + step < 16; r += 2 * step) e[r] += e[r + step];
-                part[tm] = e[0];
+                    for (int r = 0; r < 16; ++r) {
+                        const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
+                        mn = fmaxf(mn, x);
+                        if (want == tm * 16 + r) xt[tn] = x;
+                    }
+                const float ml2s = mn * kLog2e;
+#pragma unroll
+                for (int tm = 0; tm < 4; ++tm) {
+                    float e[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
+                        e[r] = fast_exp2(fmaf(x, kLog2e, -ml2s));
+                    }
+#pragma unroll
+                    for (int step = 1; step < 16; step <<= 1)
+#pragma unroll
+                        for (int r = 0; r + step < 16; r += 2 * step) e[r] += e[r + step];
+                    part[tm] = e[0];
+                }
             }
+            const float ml2n = mn * kLog2e;
             // difference of the two stored products: recomputing m_run * log2e here could be fused into an
             // FMA against ml2n and return the rounding residue of a 1e30-sized product instead of 0
             const float rescale = fast_exp2(ml2_run[tn] - ml2n);
