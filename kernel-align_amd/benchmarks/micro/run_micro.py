@@ -1,6 +1,6 @@
 """Build and run the hardware micro-benchmarks next to this file (hipcc, gfx950).
 
-    python kernel-align_amd/benchmarks/micro/run_micro.py [hbm_read_ceiling|mfma_peak|lds_read_patterns|l2_read_bandwidth|lmhead_copy_overlap ...]
+    python kernel-align_amd/benchmarks/micro/run_micro.py [hbm_read_ceiling|mfma_peak|hbm_rmw_ceiling|lds_read_patterns|l2_read_bandwidth|lmhead_copy_overlap ...]
 
 They measure the ceilings the kernels are discussed against: the pure HBM read stream, the bf16 MFMA
 peak of the instruction itself, ds_read_b128 throughput per LDS swizzle, L2 -> CU bandwidth, and how far the
