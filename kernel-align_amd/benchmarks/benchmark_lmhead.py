@@ -43,6 +43,8 @@ def main() -> int:
     ap.add_argument("--vocab", type=int, default=128256)
     ap.add_argument("--iters", type=int, default=5)
     ap.add_argument("--skip-unfused", action="store_true", help="time only the fused kernel")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the chunked backward (dhidden, dweight): 3 GEMMs of the forward's size")
     args = ap.parse_args()
 
     import torch
@@ -74,6 +76,13 @@ def main() -> int:
         ms_g = timed(gemm_only, max(2, args.iters // 2))
         out.update({"unfused_ms": ms_u, "torch_matmul_ms": ms_g, "torch_matmul_tflops": flop / ms_g / 1e9,
                     "unfused_logits_bytes": chunk * args.vocab * 2})
+    if args.backward:
+        grad = torch.randn(args.rows, generator=g, device="cuda")
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        ms_b = timed(lambda: sampler.fused_linear_logp_backward(hidden, weight, ids, grad), max(2, args.iters // 2), warmup=1)
+        out.update({"backward_ms": ms_b, "backward_tflops": 3.0 * flop / ms_b / 1e9,
+                    "backward_peak_extra_bytes": torch.cuda.max_memory_allocated() - before})
     print(json.dumps(out))
     return 0
 

@@ -65,6 +65,9 @@ class SamplerBackend(nn.Module):
     # ------------------------------------------------------------------ logprob
     @torch.inference_mode()
     def compute_logp(self, logits, token_ids, out_dtype=torch.float32, chunk_tokens=None):
+        return self._compute_logp(logits, token_ids, out_dtype, chunk_tokens)
+
+    def _compute_logp(self, logits, token_ids, out_dtype=torch.float32, chunk_tokens=None):
         """Per-token log-probabilities ``log_softmax(logits, -1)[..., token_ids]``.
 
         logits: [G, L, V] (or [N, V]) bf16 / fp16 / fp32 on the GPU; token_ids: integer tensor of
@@ -131,6 +134,9 @@ class SamplerBackend(nn.Module):
 
     @torch.inference_mode()
     def compute_logp_backward(self, logits, token_ids, logp, grad_logp, inplace=False, chunk_tokens=None):
+        return self._compute_logp_backward(logits, token_ids, logp, grad_logp, inplace, chunk_tokens)
+
+    def _compute_logp_backward(self, logits, token_ids, logp, grad_logp, inplace=False, chunk_tokens=None):
         """Gradient of ``compute_logp`` with respect to the logits, in the logits' dtype.
 
         ``dlogits[..., v] = grad_logp[...] * ((v == token_id) - softmax(logits)[..., v])``.  ``logp`` is the
@@ -254,6 +260,9 @@ class SamplerBackend(nn.Module):
     # ---------------------------------------------------------------- fused GEMM
     @torch.inference_mode()
     def fused_linear_logp(self, hidden, weight, token_ids):
+        return self._fused_linear_logp(hidden, weight, token_ids)
+
+    def _fused_linear_logp(self, hidden, weight, token_ids):
         """``compute_logp(hidden @ weight.T, token_ids)`` without materialising the logits.
 
         hidden: bf16 [..., H]; weight: bf16 [V, H] (nn.Linear.weight layout); token_ids: integer
@@ -286,3 +295,49 @@ class SamplerBackend(nn.Module):
                 ws.data_ptr(), ws_bytes, stream)
         _hip.check(status, "ka_lmhead_logprob_bf16")
         return out.view(tuple(hidden.shape[:-1]))
+
+    @torch.inference_mode()
+    def fused_linear_logp_backward(self, hidden, weight, token_ids, grad_logp, chunk_tokens=None,
+                                   dweight_dtype=torch.float32):
+        return self._fused_linear_logp_backward(hidden, weight, token_ids, grad_logp, chunk_tokens, dweight_dtype)
+
+    def _fused_linear_logp_backward(self, hidden, weight, token_ids, grad_logp, chunk_tokens=None,
+                                    dweight_dtype=torch.float32):
+        """Gradients of ``fused_linear_logp`` with respect to hidden and weight, one token chunk at a time.
+
+        Per chunk of ``chunk_tokens`` rows: the chunk's logits are rebuilt with the library bf16 GEMM, turned into
+        their gradient in place by the logprob forward + backward kernels, and contracted with weight
+        (``dhidden``) and with the chunk's hidden rows (``dweight``, accumulated over chunks in
+        ``dweight_dtype``).  Only one chunk of logits ([chunk_tokens, V] bf16) exists at any time.
+        Returns ``(dhidden [..., H] bf16, dweight [V, H] dweight_dtype)``.
+        """
+        _require_gpu(hidden, "hidden")
+        _require_gpu(weight, "weight")
+        if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            raise TypeError("fused_linear_logp_backward takes bf16 hidden and weight")
+        if weight.dim() != 2 or hidden.shape[-1] != weight.shape[1]:
+            raise ValueError("weight must be [V, H] with H == hidden.shape[-1]")
+        lead = tuple(hidden.shape[:-1])
+        if tuple(token_ids.shape) != lead or tuple(grad_logp.shape) != lead:
+            raise ValueError("token_ids and grad_logp must have shape hidden.shape[:-1]")
+        hdim = hidden.shape[-1]
+        h2 = hidden.contiguous().view(-1, hdim)
+        w2 = weight.contiguous()
+        n_rows = h2.shape[0]
+        ids = token_ids.to(device=hidden.device, dtype=torch.int64).contiguous().view(-1)
+        g = grad_logp.to(device=hidden.device, dtype=torch.float32).contiguous().view(-1)
+        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
+        if chunk < 1:
+            raise ValueError("chunk_tokens must be >= 1")
+        dhidden = torch.empty_like(h2)
+        dweight = torch.zeros(w2.shape, dtype=dweight_dtype, device=weight.device)
+        for start in range(0, n_rows, chunk):
+            stop = min(start + chunk, n_rows)
+            logits = torch.matmul(h2[start:stop], w2.t())                       # [n, V] bf16, fp32 accumulation
+            logp = self._compute_logp(logits, ids[start:stop])
+            self._compute_logp_backward(logits, ids[start:stop], logp, g[start:stop], inplace=True)
+            torch.matmul(logits, w2, out=dhidden[start:stop])                   # logits now holds dlogits
+            part = torch.matmul(logits.t(), h2[start:stop])                     # [V, H] bf16
+            dweight.add_(part)
+            del logits, part
+        return dhidden.view(hidden.shape), dweight

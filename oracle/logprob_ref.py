@@ -111,3 +111,24 @@ def logprob_backward_closed_form(logits: torch.Tensor, token_ids: torch.Tensor, 
     p = torch.softmax(x, dim=-1)
     onehot = torch.zeros_like(p).scatter_(-1, token_ids.cpu().to(torch.int64).unsqueeze(-1), 1.0)
     return grad_logp.detach().cpu().double().unsqueeze(-1) * (onehot - p)
+
+
+def lmhead_logprob_backward_ref(hidden: torch.Tensor, weight: torch.Tensor, token_ids: torch.Tensor,
+                                grad_logp: torch.Tensor, dtype=torch.float64):
+    """(dhidden, dweight) of lmhead_logprob_ref by torch autograd on the CPU in `dtype`: the gradient of
+    compute_logp(lm_head(hidden)) (rl_engine/kernels/sampling.py:108-110 behind an nn.Linear)."""
+    h = hidden.detach().cpu().to(dtype).clone().requires_grad_(True)
+    w = weight.detach().cpu().to(dtype).clone().requires_grad_(True)
+    logits = torch.nn.functional.linear(h, w)
+    lp = torch.log_softmax(logits, dim=-1).gather(-1, token_ids.cpu().to(torch.int64).unsqueeze(-1)).squeeze(-1)
+    lp.backward(grad_logp.detach().cpu().to(dtype))
+    return h.grad, w.grad
+
+
+def lmhead_logprob_backward_closed_form(hidden: torch.Tensor, weight: torch.Tensor, token_ids: torch.Tensor,
+                                        grad_logp: torch.Tensor):
+    """The same two gradients written out in fp64: D = g * (onehot - softmax(h W^T)); dh = D W; dW = D^T h."""
+    h = hidden.detach().cpu().double().reshape(-1, hidden.shape[-1])
+    w = weight.detach().cpu().double()
+    d = logprob_backward_closed_form(h @ w.t(), token_ids.reshape(-1), grad_logp.reshape(-1))
+    return (d @ w).reshape(hidden.shape), d.t() @ h

@@ -1,0 +1,71 @@
+"""The differentiable wrappers (rl_engine.kernels.autograd) and the chunked lm_head backward against fp64
+autograd / closed forms on the CPU.  Needs an MI355X.
+
+Tolerances: logp_from_logits returns its gradient in the logits' dtype (bf16: relative 2^-8).  The lm_head
+backward rebuilds bf16 logits and bf16 logit gradients before two bf16 GEMMs, so its results carry bf16
+rounding of three intermediates: compared by relative Frobenius error, 2e-2.
+"""
+import pytest
+import torch
+
+from oracle import logprob_ref as O
+from rl_engine.kernels.autograd import linear_logp, logp_from_logits
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(got, want):
+    return ((got.double().cpu() - want).norm() / want.norm()).item()
+
+
+def test_logp_from_logits_backward_matches_autograd(sampler):
+    g = torch.Generator().manual_seed(0)
+    logits = (torch.randn(3, 17, 2056, generator=g) * 3).bfloat16()
+    ids = torch.randint(0, 2056, (3, 17), generator=g)
+    w = torch.randn(3, 17, generator=g)
+    x = logits.cuda().requires_grad_(True)
+    lp = logp_from_logits(sampler, x, ids.cuda())
+    assert lp.requires_grad and lp.dtype == torch.float32
+    (lp * w.cuda()).sum().backward()
+    want = O.logprob_backward_closed_form(logits, ids, w)
+    err = (x.grad.double().cpu() - want).abs()
+    assert (err <= 2.0 ** -8 * want.abs() + 1e-6).all()
+    assert torch.allclose(lp.detach().cpu(), O.logprob_ref(logits, ids), atol=1e-4, rtol=0)
+
+
+@pytest.mark.parametrize("n,h,v,chunk", [(300, 256, 1000, None), (300, 256, 1000, 128), (64, 128, 4099, 50)])
+def test_linear_logp_backward(sampler, n, h, v, chunk):
+    g = torch.Generator().manual_seed(n + v)
+    hidden = torch.randn(n, h, generator=g).bfloat16()
+    weight = (torch.randn(v, h, generator=g) * 0.05).bfloat16()
+    ids = torch.randint(0, v, (n,), generator=g)
+    w = torch.randn(n, generator=g)
+    hx = hidden.cuda().requires_grad_(True)
+    wx = weight.cuda().requires_grad_(True)
+    lp = linear_logp(sampler, hx, wx, ids.cuda(), chunk_tokens=chunk)
+    (lp * w.cuda()).sum().backward()
+    dh_ref, dw_ref = O.lmhead_logprob_backward_ref(hidden, weight, ids, w)
+    dh_cf, dw_cf = O.lmhead_logprob_backward_closed_form(hidden, weight, ids, w)
+    assert rel_err(dh_cf, dh_ref) < 1e-10 and rel_err(dw_cf, dw_ref) < 1e-10   # the oracle's two forms agree
+    assert hx.grad.dtype == torch.bfloat16 and wx.grad.dtype == torch.bfloat16
+    assert rel_err(hx.grad, dh_ref) < 2e-2
+    assert rel_err(wx.grad, dw_ref) < 2e-2
+    assert torch.allclose(lp.detach().cpu(), O.lmhead_logprob_ref(hidden, weight, ids), atol=2e-2, rtol=0)
+
+
+def test_chunked_backward_direct_call_and_shapes(sampler):
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(2, 40, 192, generator=g).bfloat16().cuda()
+    weight = (torch.randn(777, 192, generator=g) * 0.05).bfloat16().cuda()
+    ids = torch.randint(0, 777, (2, 40), generator=g).cuda()
+    grad = torch.randn(2, 40, generator=g).cuda()
+    dh, dw = sampler.fused_linear_logp_backward(hidden, weight, ids, grad, chunk_tokens=32)
+    assert dh.shape == hidden.shape and dh.dtype == torch.bfloat16
+    assert dw.shape == weight.shape and dw.dtype == torch.float32
+    dh_ref, dw_ref = O.lmhead_logprob_backward_ref(hidden.reshape(-1, 192), weight, ids.reshape(-1), grad.reshape(-1))
+    assert rel_err(dh.reshape(-1, 192), dh_ref.reshape(-1, 192)) < 2e-2
+    assert rel_err(dw, dw_ref) < 2e-2
+    with pytest.raises(ValueError):
+        sampler.fused_linear_logp_backward(hidden, weight, ids[:1], grad)
+    with pytest.raises(TypeError):
+        sampler.fused_linear_logp_backward(hidden.float(), weight, ids, grad)

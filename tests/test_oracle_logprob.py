@@ -117,3 +117,31 @@ def test_backward_closed_form_is_autograd():
         xp[r, c] += eps
         fd = ((O.logprob_f64(xp, i2) * g2).sum() - base) / eps
         assert abs(fd.item() - an[r, c].item()) < 1e-5
+
+
+def test_lmhead_backward_oracle_forms_agree_and_match_finite_differences():
+    """Autograd and the written-out D W / D^T h agree; a central difference of the fp64 forward pins both
+    against a transposed operand or a dropped one-hot term."""
+    g = torch.Generator().manual_seed(11)
+    hidden = torch.randn(6, 16, generator=g).bfloat16()
+    weight = (torch.randn(23, 16, generator=g) * 0.3).bfloat16()
+    ids = torch.randint(0, 23, (6,), generator=g)
+    grad = torch.randn(6, generator=g)
+    dh_a, dw_a = O.lmhead_logprob_backward_ref(hidden, weight, ids, grad)
+    dh_c, dw_c = O.lmhead_logprob_backward_closed_form(hidden, weight, ids, grad)
+    assert torch.allclose(dh_a, dh_c, atol=1e-12) and torch.allclose(dw_a, dw_c, atol=1e-12)
+
+    def loss(h, w):
+        lp = torch.log_softmax(h @ w.t(), -1).gather(-1, ids.unsqueeze(-1)).squeeze(-1)
+        return (lp * grad.double()).sum()
+
+    h0, w0 = hidden.double(), weight.double()
+    eps = 1e-6
+    for (r, c) in [(0, 0), (3, 7), (5, 15)]:
+        e = torch.zeros_like(h0); e[r, c] = eps
+        fd = (loss(h0 + e, w0) - loss(h0 - e, w0)) / (2 * eps)
+        assert abs(fd.item() - dh_c[r, c].item()) < 1e-7
+    for (r, c) in [(0, 0), (int(ids[2]), 3), (22, 15)]:
+        e = torch.zeros_like(w0); e[r, c] = eps
+        fd = (loss(h0, w0 + e) - loss(h0, w0 - e)) / (2 * eps)
+        assert abs(fd.item() - dw_c[r, c].item()) < 1e-7
