@@ -151,7 +151,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-sample-rows", type=int, default=32768,
+    ap.add_argument("--cpu-sample-rows", type=int, default=131072,
                     help="rows of the tensor the CPU oracle is timed on (0 = skip)")
     ap.add_argument("--chunk-tokens", type=int, default=None, help="rows per kernel launch")
     ap.add_argument("--skip-lmhead", action="store_true", help="leave the fused lm_head->logprob figure out")

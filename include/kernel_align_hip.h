@@ -108,6 +108,7 @@ int ka_logprob_backward_f32(const void *logits, int64_t n_rows, int64_t vocab, i
  * 2^-40 fixed point, then summed as integers, so the result does not depend on
  * summation order, batch size or launch geometry.
  * uniforms: one fp32 in [0,1) per row.  out_ids: int64 [batch].
+ * A NaN logit counts as -inf; a row with nothing above -inf is sampled uniformly.
  */
 size_t ka_sample_workspace_bytes(int64_t batch, int64_t vocab);
 int ka_sample_topk_topp_bf16(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,

@@ -125,6 +125,7 @@ __device__ __forceinline__ uint32_t elem_key(typename T::raw_t raw, float temp, 
     float y = T::widen(raw);
     if (has_t) y = Round<T>::apply(y / temp);
     y = (y == 0.0f) ? 0.0f : y;
+    y = (y != y) ? -__builtin_inff() : y;  // a NaN logit counts as -inf: it is never preferred to a number
     return masked_key<T>(y);
 }
 
@@ -381,6 +382,9 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         if (guard == 64) return false;  // a huge temperature folds many values together: radix path
     }
     const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
+    // Fewer than top_k lanes hold a number above -inf: the survivors then include -inf entries (and NaNs,
+    // which count as -inf but fail every float compare).  Leave such rows to the radix path.
+    if (boundf == -__builtin_inff()) return false;
     auto collect = [&](int i, typename T::raw_t raw) {
         if (T::widen(raw) >= boundf) {
             const uint32_t slot = atomicAdd(&sh.n_cand, 1u);

@@ -222,6 +222,7 @@ int ka_oracle_sample(const void *logits, int dtype, int64_t batch, int64_t vocab
         float mx = -INFINITY;
         for (int64_t i = 0; i < vocab; ++i) {
             y[i] = load_scaled(row, dtype, i, temperature);
+            if (y[i] != y[i]) y[i] = -INFINITY; /* a NaN logit counts as -inf (the reference would fail on it) */
             keys[i] = key_of(y[i]);
             if (i == 0 || keys[i] > key_of(mx)) mx = y[i];
         }

@@ -187,3 +187,20 @@ def test_baseline_sampling_config_agrees_exactly():
     a = exact.sample(logits, 0.7, 50, 0.9, u)
     b, margin = sampling_ref.sample(logits, 50, 0.9, 0.7, u)
     assert torch.equal(a, b) and margin.min().item() > 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_nan_logits_count_as_minus_infinity(dtype):
+    """The convention for inputs the reference cannot take: a row with NaNs samples exactly like the
+    same row with -inf in their place, and a NaN entry is never drawn while a number is available."""
+    g = torch.Generator().manual_seed(41)
+    logits = (torch.randn(16, 700, generator=g) * 3).to(dtype)
+    holes = torch.rand(16, 700, generator=g) < 0.2
+    with_nan = logits.clone(); with_nan[holes] = float("nan")
+    with_inf = logits.clone(); with_inf[holes] = float("-inf")
+    u = torch.rand(16, generator=g)
+    for k, p, temp in [(50, 0.9, 0.7), (None, None, 1.0), (600, 0.99, 1.5), (None, 0.5, 1.0)]:
+        a = exact.sample(with_nan, temp, k, p, u)
+        b = exact.sample(with_inf, temp, k, p, u)
+        assert torch.equal(a, b)
+        assert not holes[torch.arange(16), a].any()

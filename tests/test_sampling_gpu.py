@@ -219,3 +219,30 @@ def test_per_row_parameters_and_sampled_logprob(sampler, dtype, monkeypatch):
     # the log-probability is the one of the filtered distribution: top_k = 1 -> log 1 = 0 without ties
     _, lp_greedy = sampler.sample(torch.randn(8, 1000, generator=g).cuda(), top_k=1, uniforms=u[:8].cuda(), return_logprob=True)
     assert (lp_greedy == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_nan_and_infinite_logits_on_both_paths(sampler, dtype, monkeypatch):
+    """NaN counts as -inf, +inf takes all the mass, rows with fewer than top_k numbers above -inf keep their
+    -inf entries: same ids from the candidate-list path, the radix path and the oracle."""
+    g = torch.Generator().manual_seed(43)
+    base = (torch.randn(24, 5000, generator=g) * 3).to(dtype)
+    holes = torch.rand(24, 5000, generator=g) < 0.3
+    nan_rows = base.clone(); nan_rows[holes] = float("nan")
+    sparse = torch.full((24, 5000), float("-inf")).to(dtype)            # 10 numbers per row, the rest masked / NaN
+    cols = torch.randint(0, 5000, (24, 10), generator=g)
+    sparse.scatter_(1, cols, (torch.randn(24, 10, generator=g) * 2).to(dtype))
+    sparse[:, ::7] = torch.where(torch.isinf(sparse[:, ::7].float()), torch.tensor(float("nan")).to(dtype), sparse[:, ::7])
+    pinf = base.clone(); pinf[:, 123] = float("inf"); pinf[::2, 4000] = float("inf")
+    allnan = torch.full((4, 5000), float("nan")).to(dtype)
+    u = torch.rand(24, generator=g)
+    for logits, k, p, temp in [(nan_rows, 50, 0.9, 0.7), (nan_rows, None, 0.8, 1.0), (sparse, 50, 0.9, 0.7),
+                               (sparse, 5, None, 1.3), (pinf, 50, 0.9, 0.7), (pinf, None, None, 1.0),
+                               (allnan, 50, 0.9, 0.7)]:
+        uu = u[:logits.shape[0]]
+        want = exact.sample(logits, temp, k, p, uu)
+        for radix_only in ("0", "1"):
+            monkeypatch.setenv("KA_SAMPLE_RADIX_ONLY", radix_only)
+            got = run(sampler, logits, uu, k, p, temp)
+            assert torch.equal(got, want), f"radix_only={radix_only} k={k} p={p} T={temp}"
+        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
