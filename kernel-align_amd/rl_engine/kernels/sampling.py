@@ -12,7 +12,7 @@ import torch
 import torch.nn as nn
 
 from rl_engine.kernels import _hip
-from rl_engine.kernels.pool import WorkspacePool
+from rl_engine.kernels.pool import PoolExhausted, WorkspacePool
 from rl_engine.platforms.constants import constants
 from rl_engine.utils.logger import logger
 
@@ -285,15 +285,25 @@ class SamplerBackend(nn.Module):
         out = torch.empty(n_rows, dtype=torch.float32, device=hidden.device)
         if n_rows == 0:
             return out.view(tuple(hidden.shape[:-1]))
-        ws_bytes = self._lib.ka_lmhead_workspace_bytes(n_rows, hdim, vocab)
-        self.pool.reset()
-        ws = self.pool.reserve(ws_bytes, hidden.device)
+        # The workspace holds 16 B per row and vocabulary split; rows go to the kernel in slices that fit
+        # the pool (a multiple of the 256-token tile), which does not change any row's result.
+        per_row = self._lib.ka_lmhead_workspace_bytes(256, hdim, vocab) // 256
+        fit = self.pool.capacity // max(per_row, 1)
+        rows_per_call = n_rows if n_rows <= fit else fit // 256 * 256
+        if rows_per_call < 1:
+            raise PoolExhausted(f"the {self.pool.capacity} B pool cannot hold the lm_head partials of one "
+                                f"256-token tile ({256 * per_row} B)")
         with torch.cuda.device(hidden.device):
             stream = torch.cuda.current_stream().cuda_stream
-            status = self._lib.ka_lmhead_logprob_bf16(
-                h2.data_ptr(), w2.data_ptr(), ids.data_ptr(), out.data_ptr(), n_rows, hdim, vocab,
-                ws.data_ptr(), ws_bytes, stream)
-        _hip.check(status, "ka_lmhead_logprob_bf16")
+            for start in range(0, n_rows, rows_per_call):
+                n = min(rows_per_call, n_rows - start)
+                ws_bytes = self._lib.ka_lmhead_workspace_bytes(n, hdim, vocab)
+                self.pool.reset()
+                ws = self.pool.reserve(ws_bytes, hidden.device)
+                status = self._lib.ka_lmhead_logprob_bf16(
+                    h2.data_ptr() + start * hdim * 2, w2.data_ptr(), ids.data_ptr() + start * 8,
+                    out.data_ptr() + start * 4, n, hdim, vocab, ws.data_ptr(), ws_bytes, stream)
+                _hip.check(status, "ka_lmhead_logprob_bf16")
         return out.view(tuple(hidden.shape[:-1]))
 
     @torch.inference_mode()

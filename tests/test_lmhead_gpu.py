@@ -66,3 +66,19 @@ def test_bit_identical_across_runs_and_row_counts(sampler):
     for n in (1, 255, 256, 1024):
         assert torch.equal(base[:n], sampler.fused_linear_logp(h[:n], w, i[:n]))
     assert torch.equal(base[600:900], sampler.fused_linear_logp(h[600:900], w, i[600:900]))
+
+
+def test_rows_are_sliced_to_fit_a_small_workspace_pool(sampler):
+    """With a pool too small for all rows the wrapper feeds the kernel 256-row multiples; the result is
+    bit-identical to the single call (every row's reduction order is fixed)."""
+    from rl_engine.kernels.pool import PoolExhausted
+    from rl_engine.kernels.sampling import SamplerBackend
+
+    hidden, weight, ids = make(1000, 128, 40000, seed=9)                # 3 vocabulary splits: 48 B per row
+    base = sampler.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
+    small = SamplerBackend(pool_bytes=300 * 48).cuda()                   # room for 300 rows -> slices of 256
+    assert torch.equal(small.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda()), base)
+    tiny = SamplerBackend(pool_bytes=100 * 48).cuda()                    # less than one tile of a long input
+    with pytest.raises(PoolExhausted):
+        tiny.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
+    assert torch.equal(tiny.fused_linear_logp(hidden[:64].cuda(), weight.cuda(), ids[:64].cuda()), base[:64])
