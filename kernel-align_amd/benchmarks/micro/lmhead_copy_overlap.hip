@@ -5,14 +5,14 @@
 //   - the slab's 64 MFMAs alone (32x32x16 bf16 on registers; no fragment reads, one barrier per slab);
 //   - both, with the copies running LOOK slabs ahead of the one consumed (LOOK = 1 is what two 64 KB stages in
 //     LDS allow: nothing is in flight at the moment a slab is waited for; LDS contents are garbage here, so deeper
-//     lookahead can be timed although it would not fit).
+//     lookahead can be timed although it would not fit; "1.5 slabs" = five 32 KB half-slab buffers, which do fit).
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 typedef __attribute__((address_space(3))) void lds_void;
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-template <int LOOK, bool COPY, bool MFMA>
+template <int LOOK, bool COPY, bool MFMA, bool HALF = false, bool LEAN = false>
 __global__ __launch_bounds__(256) void k(const char *__restrict__ W, const char *__restrict__ H, int n_splits,
                                          int tiles_per_split, int nk, unsigned *out) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -25,27 +25,45 @@ __global__ __launch_bounds__(256) void k(const char *__restrict__ W, const char 
     const char *hb = H + size_t(tb) * 256 * 8192;
     const unsigned lane_off = unsigned(wave * 8 + (lane >> 3)) * 8192 + (lane & 7) * 16;
     const int steps = tiles_per_split * nk;
+    // LEAN: a wavefront-uniform base (SGPRs) plus eight lane offsets computed once, so that a copy costs no
+    // vector arithmetic at all.
+    unsigned voff[8];
+    for (int j = 0; j < 8; ++j) voff[j] = lane_off + j * 32 * 8192;
     auto issue1 = [&](int s, int c) {
         if (s >= steps) s = steps - 1;
         const int vt = s / nk, kt = s % nk;
+        if (LEAN) {
+            const char *base = ((c & 1) ? hb : wb + size_t(vt) * 256 * 8192) + kt * 128;
+            unsigned char *dst = lds + (s & 1) * 65536 + wave * 1024 + (c & 1) * 32768 + (c >> 1) * 4096;
+            __builtin_amdgcn_global_load_lds(base + voff[c >> 1], (lds_void *)dst, 16, 0, 0);
+            return;
+        }
         const char *src = ((c & 1) ? hb : wb + size_t(vt) * 256 * 8192) + kt * 128 + lane_off + (c >> 1) * 32 * 8192;
         unsigned char *dst = lds + (s & 1) * 65536 + wave * 1024 + (c & 1) * 32768 + (c >> 1) * 4096;
         __builtin_amdgcn_global_load_lds(src, (lds_void *)dst, 16, 0, 0);
     };
-    if (COPY)
+    if (COPY) {
         for (int s = 0; s < LOOK; ++s)
 #pragma unroll
             for (int c = 0; c < 16; ++c) issue1(s, c);
+        if (HALF)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) issue1(LOOK, c);
+    }
     f32x16 acc[16];
     for (int i = 0; i < 16; ++i)
         for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
     bf16x8 fa, fb;
     for (int i = 0; i < 8; ++i) { fa[i] = (__bf16)float(lane + i); fb[i] = (__bf16)float(lane - i); }
     for (int s = 0; s < steps; ++s) {
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(16 * (LOOK - 1)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(16 * (LOOK - 1) + (HALF ? 8 : 0)) : "memory");
 #pragma unroll
         for (int g = 0; g < 32; ++g) {  // one copy per pair of MFMAs in the first half of the slab
-            if (COPY && g < 16) issue1(s + LOOK, g);
+            if (COPY && g < 16) {
+                if (!HALF) issue1(s + LOOK, g);
+                else if (g < 8) issue1(s + LOOK, 8 + g);  // second half of slab s + LOOK, then first half of the one after
+                else issue1(s + LOOK + 1, g - 8);
+            }
             if (MFMA) {
                 acc[(2 * g) & 15] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc[(2 * g) & 15], 0, 0, 0);
                 acc[(2 * g + 1) & 15] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb, fa, acc[(2 * g + 1) & 15], 0, 0, 0);
@@ -99,6 +117,10 @@ int main() {
     run("copies alone, 3 slabs ahead", k<3, true, false>, true, false);
     run("MFMAs alone (barrier per slab)", k<1, false, true>, false, true);
     run("copies + MFMAs, 1 slab ahead", k<1, true, true>, true, true);
+    run("copies + MFMAs, 1.5 slabs ahead (5 x 32 KB)", k<1, true, true, true>, true, true);
+    run("copies alone, 1.5 slabs ahead", k<1, true, false, true>, true, false);
+    run("lean addressing: copies + MFMAs, 1 slab ahead", k<1, true, true, false, true>, true, true);
+    run("lean addressing: copies + MFMAs, 1.5 slabs", k<1, true, true, true, true>, true, true);
     run("copies + MFMAs, 2 slabs ahead", k<2, true, true>, true, true);
     run("copies + MFMAs, 3 slabs ahead", k<3, true, true>, true, true);
     return 0;
