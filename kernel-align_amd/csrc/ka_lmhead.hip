@@ -7,7 +7,8 @@
 //     slabs of 64 (one cache line per row); the W slab [256 x 64] and the hidden
 //     slab [256 x 64] go from global memory straight into XOR-swizzled LDS
 //     (global_load_lds_dwordx4, no register staging), two stages of 64 KB, one
-//     barrier per slab; fragment reads run one k-step ahead of the MFMAs;
+//     barrier per slab, three quarters into it; fragment reads run one k-step
+//     ahead of the MFMAs;
 //   * the MFMA "A" operand is W (rows of the result = vocabulary entries) and
 //     "B" is hidden (columns = tokens), so every lane's 64 accumulators of one
 //     32-column block belong to ONE token: the online max / sum-of-exp update
@@ -400,8 +401,9 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     if (grid >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "lmhead: grid too large");
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     Partial *partials = static_cast<Partial *>(workspace);
-    static const hipError_t attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials),
-                                                          hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
+    // set on every call rather than once per process: the attribute belongs to the current device
+    const hipError_t attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
     if (attr_rc != hipSuccess) return check_hip(attr_rc, "lmhead: reserving 128 KB of LDS");
     hipLaunchKernelGGL(lmhead_partials, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                        static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
