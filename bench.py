@@ -62,7 +62,7 @@ def cpu_baseline(logits, ids, sample_rows: int):
     }
 
 
-def sampling_latency(sampler, steps: int, warmup: int):
+def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
     """Fused sampling on bf16 [B, 128256], T=0.7, top-k 50, top-p 0.9, uniforms from seed 1234."""
     import torch
     from benchmarks.workloads import cfg5_sampling
@@ -89,6 +89,26 @@ def sampling_latency(sampler, steps: int, warmup: int):
             gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel": "sample_rows<Bf16>"}
+            if cpu:
+                # The torch restatement of the reference's native_sampling and the exact C definition, timed on
+                # the host on the same rows (median of 3); both also check the ids of the GPU run.
+                from oracle import exact, sampling_ref
+                got = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u).cpu()
+                lc, uc = logits.cpu(), u.cpu()
+                times = {"torch_restatement": [], "exact_c": []}
+                for _ in range(3):
+                    t0 = time.perf_counter()
+                    want_t, _ = sampling_ref.sample(lc, top_k=50, top_p=0.9, temperature=0.7, uniforms=uc)
+                    times["torch_restatement"].append(time.perf_counter() - t0)
+                    t0 = time.perf_counter()
+                    want_c = exact.sample(lc, 0.7, 50, 0.9, uc)
+                    times["exact_c"].append(time.perf_counter() - t0)
+                out["cpu_baseline"] = {
+                    "unit": "ms", "batch": batch, "cores": torch.get_num_threads(), "kind": "port",
+                    "torch_restatement_ms": sorted(times["torch_restatement"])[1] * 1e3,
+                    "exact_c_ms_single_thread": sorted(times["exact_c"])[1] * 1e3,
+                    "ids_equal_exact": bool(torch.equal(got, want_c)),
+                    "ids_equal_torch_restatement": bool(torch.equal(got, want_t.to(got.dtype).view(-1)))}
     return out
 
 
@@ -246,7 +266,7 @@ def main() -> int:
     del logits3, ids2, logits, ids
     torch.cuda.empty_cache()
     result["logprob_backward"] = backward_throughput(sampler)
-    result["sampling"] = sampling_latency(sampler, args.steps, args.warmup)
+    result["sampling"] = sampling_latency(sampler, args.steps, args.warmup, cpu=args.cpu_sample_rows > 0)
     if not args.skip_lmhead:
         result["fused_lm_head"] = lmhead_throughput(sampler)
     print(json.dumps(result), flush=True)
