@@ -89,6 +89,22 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
             gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel": "sample_rows<Bf16>"}
+            # the other filter combinations at the same batch (kernel time per call, microseconds)
+            modes = {}
+            for name, kw in (("no_filter_T1", dict(temperature=1.0)), ("no_filter_T0.7", dict(temperature=0.7)),
+                             ("top_p0.9_T0.7", dict(top_p=0.9, temperature=0.7)),
+                             ("top_k2000_top_p0.9_T0.7", dict(top_k=2000, top_p=0.9, temperature=0.7)),
+                             ("top_k50_T0.7", dict(top_k=50, temperature=0.7))):
+                for _ in range(3):
+                    sampler.sample(logits, uniforms=u, **kw)
+                torch.cuda.synchronize()
+                ev0.record()
+                for _ in range(20):
+                    sampler.sample(logits, uniforms=u, **kw)
+                ev1.record()
+                torch.cuda.synchronize()
+                modes[name] = ev0.elapsed_time(ev1) / 20 * 1e3
+            out["other_modes_us_b256"] = modes
             if cpu:
                 # The torch restatement of the reference's native_sampling and the exact C definition, timed on
                 # the host on the same rows (median of 3); both also check the ids of the GPU run.

@@ -140,6 +140,15 @@ int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, in
                  float *out_logprob, void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
+ * The integer mass function of the sampling operator, element-wise: out[i] = W(d[i]) =
+ * trunc(2^40 * exp(d[i])) for d <= 0 (W(0) = 2^40, 0 once d * log2(e) < -41), evaluated by the fixed
+ * operation sequence the sampling kernels use.  Exported so that the function every sampled id depends on
+ * can be checked bit for bit against its CPU statement; no counterpart in the reference, whose masses are
+ * torch.softmax values (benchmarks/benchmark_sampling.py:27,36).
+ */
+int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, void *hip_stream);
+
+/*
  * Fused lm_head -> logprob without materialised logits:
  *     out[r] = h_r . W[ids[r]] - logsumexp_v(h_r . W[v])               (fp32)
  * hidden: bf16 [n_rows, hidden_dim] row-major; weight: bf16 [vocab, hidden_dim]

@@ -44,28 +44,31 @@ template <typename T> __device__ __forceinline__ float value_of(uint32_t key) {
     return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : (~key & key_mask<T>()));
 }
 
-// W(d) = trunc(2^40 * exp(d)), d <= 0.  Separate IEEE multiplies and adds (the
-// _rn intrinsics are never contracted into FMAs), Taylor coefficients 1/k!.
+// W(d) = trunc(2^40 * exp(d)), d <= 0, by a fixed sequence of IEEE double operations: one multiply for the
+// range reduction, a degree-11 Horner evaluation with fused multiply-adds (Taylor coefficients 1/k!), one
+// multiply by a power of two.  Contraction is off in this function, so exactly the operations written here
+// are executed (the CPU statement of the operator performs the same ones, fma() included).  No branches: this
+// runs for up to every entry of a row.
 __device__ __forceinline__ uint64_t weight_fix(float d) {
+#pragma clang fp contract(off)
     constexpr double C[12] = {0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,
                               0x1.5555555555555p-3,  0x1.5555555555555p-5,  0x1.1111111111111p-7,
                               0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16,
                               0x1.71de3a556c734p-19, 0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26};
     constexpr double LOG2E = 0x1.71547652b82fep+0, LN2 = 0x1.62e42fefa39efp-1;
-    if (!(d <= 0.0f)) return d > 0.0f ? (uint64_t(1) << FIX_BITS) : 0;
-    const double t = __dmul_rn(double(d), LOG2E);
-    if (t < -41.0) return 0;
-    const int n = int(__dadd_rn(t, -0.5));
-    const double f = __dsub_rn(t, double(n));
-    const double g = __dmul_rn(f, LN2);
+    const double t = double(d) * LOG2E;
+    const double tc = t < -64.0 ? -64.0 : t;  // keeps the conversion below in range; such t give 0 anyway
+    const int n = int(tc - 0.5);
+    const double f = tc - double(n);
+    const double g = f * LN2;
     double p = C[11];
 #pragma unroll
-    for (int k = 10; k >= 0; --k) {
-        p = __dmul_rn(p, g);
-        p = __dadd_rn(p, C[k]);
-    }
+    for (int k = 10; k >= 0; --k) p = __builtin_fma(p, g, C[k]);
     const double scale = __longlong_as_double((long long)(uint64_t(1023 + FIX_BITS + n) << 52));
-    return (uint64_t)__dmul_rn(p, scale);
+    // trunc(p * scale) < 2^42 as an integer: the low mantissa bits of trunc(.) + 2^52
+    const uint64_t w = uint64_t(__double_as_longlong(__builtin_trunc(p * scale) + 0x1p52)) & 0x000fffffffffffffull;
+    const uint64_t special = d > 0.0f ? (uint64_t(1) << FIX_BITS) : 0ull;  // d > 0 cannot occur; NaN -> 0
+    return (d <= 0.0f && !(t < -41.0)) ? w : special;
 }
 
 // log(w / z) for integer masses, in fp64 (w >= 1: an entry of mass 0 is never drawn).
@@ -146,6 +149,17 @@ struct Candidates {            // 24 KB, same footprint as the histograms
     uint64_t w[CAND_CAP];      // integer masses in that order
 };
 
+struct DenseScalars {
+    uint64_t wave_u64[S_WAVES];
+    uint32_t wave_u32[S_WAVES];
+    uint64_t tile_mass[17];  // 16 tiles of 8192 entries + the ragged tail
+    uint32_t tile_ties[17];  // entries equal to the cut key in each tile
+    uint64_t z_topk, before_cut, w_cut, pick_w;
+    uint32_t i_topk, n_cut, kcut16;
+    int best_i;
+    int64_t hit;
+};
+
 struct alignas(16) Shared {
     union {
         Histograms h;
@@ -161,6 +175,7 @@ struct alignas(16) Shared {
     int64_t hit;
     uint32_t n_cand, pick_a, pick_b;
     uint64_t pick_z;
+    DenseScalars ds;  // scalars of the resident no-filter path
 };
 
 template <typename V> __device__ __forceinline__ V shfl_up_v(V v, int off) { return __shfl_up(v, off, kWave); }
@@ -505,6 +520,509 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     return true;
 }
 
+
+// ---------------------------------------------------------------------------
+// Resident-row paths for 16-bit dtypes (bf16, fp16), rows of at most 131,072 entries, 16-byte aligned.
+//
+// The row is read once into registers (16 x uint4 per lane) and every entry is replaced by the 16-bit
+// order-preserving key of its scaled value, so the later passes neither touch memory nor divide again.
+// Since a 16-bit dtype has only 65,536 values, an entry's integer mass is a function of its key.
+//
+//   no filter   : one pass evaluates every entry's mass and leaves the mass of each 8192-entry tile in LDS;
+//                 the draw walks tile totals, then the per-lane sums of one tile, then eight entries.
+//   dense path  : (top-p without top-k, or top_k > 1024) a count histogram over all 65,536 keys in LDS
+//                 (16-bit counters, two per word) is compacted into a list of the occupied keys in
+//                 descending order; masses are evaluated once per occupied key (a few thousand instead of
+//                 128 K), prefix sums over the list give the top-k key, Z, the top-p cut key and the
+//                 surviving mass; the masses of the surviving keys go into a table indexed by
+//                 key - cut key, and the draw runs as above with one LDS lookup per entry.
+// Both return false (having written no output) when a row does not fit (not resident, a counter overflow, too
+// many occupied keys, survivors spanning too many keys, a top-p cut inside a tie group); the radix path then runs.
+// All integer decisions are the same function of the row as in the radix path.
+// ---------------------------------------------------------------------------
+constexpr int RES_VECS = 16;
+constexpr int D_WORDS = 32768;              // 65,536 16-bit counters
+constexpr int D_LIST_CAP = 7168;            // occupied keys the list can hold (4 B each)
+constexpr int D_TABLE_CAP = D_LIST_CAP / 2; // keys spanned by the survivors (8 B each, same LDS region)
+constexpr int D_PER_THREAD = D_LIST_CAP / S_THREADS;  // list entries per thread
+
+constexpr size_t DENSE_LDS_BYTES = size_t(D_WORDS) * 4 + size_t(D_LIST_CAP) * 4 + sizeof(DenseScalars);
+
+template <typename T> __device__ __forceinline__ uint32_t key16_of(float y) {  // y is a value of the dtype
+    if (T::kDtype == KA_DTYPE_BF16) return masked_key<T>(y) >> 16;
+    union { _Float16 h; uint16_t u; } c;
+    c.h = _Float16(y);
+    return (c.u & 0x8000u) ? (~uint32_t(c.u) & 0xffffu) : (uint32_t(c.u) | 0x8000u);
+}
+template <typename T> __device__ __forceinline__ float value_of_key16(uint32_t k) {
+    if (T::kDtype == KA_DTYPE_BF16) return value_of<T>(k << 16);
+    union { _Float16 h; uint16_t u; } c;
+    c.u = uint16_t((k & 0x8000u) ? (k & 0x7fffu) : (~k & 0xffffu));
+    return float(c.h);
+}
+// 16-bit key of the scaled entry (temperature, -0 -> +0, NaN -> -inf), computed on the 16-bit patterns with
+// selects only: this runs once per entry of the row.
+template <typename T, bool HAS_T>
+__device__ __forceinline__ uint32_t elem_key16(uint32_t raw, float temp) {
+    uint32_t h = raw;  // 16-bit pattern of the scaled value
+    if (HAS_T) {
+        const float q = T::widen(typename T::raw_t(raw)) / temp;
+        if (T::kDtype == KA_DTYPE_BF16) {
+            const uint32_t b = __float_as_uint(q);
+            // round to nearest even on the upper 16 bits; +-inf stays, a NaN is replaced below
+            h = ((b + 0x7fffu + ((b >> 16) & 1u)) >> 16) | (((b & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : 0u);
+        } else {
+            union { _Float16 f; uint16_t u; } c;
+            c.f = _Float16(q);
+            h = c.u;
+        }
+    }
+    constexpr uint32_t kInf = T::kDtype == KA_DTYPE_BF16 ? 0x7f80u : 0x7c00u;
+    const uint32_t mag = h & 0x7fffu;
+    h = mag == 0 ? 0u : h;                        // -0 -> +0
+    h = mag > kInf ? (0x8000u | kInf) : h;        // NaN -> -inf
+    return (h & 0x8000u) ? (~h & 0xffffu) : (h | 0x8000u);
+}
+
+__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ uint32_t block_max_u32_buf(uint32_t v, uint32_t *wave_buf) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t t = __shfl_xor(v, off, kWave);
+        v = t > v ? t : v;
+    }
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) wave_buf[threadIdx.x / kWave] = v;
+    __syncthreads();
+    uint32_t r = wave_buf[0];
+#pragma unroll
+    for (int w = 1; w < S_WAVES; ++w) r = wave_buf[w] > r ? wave_buf[w] : r;
+    return r;
+}
+
+// Entry j (0..7) of a vector of eight 16-bit keys, for a j that is not a compile-time constant (register
+// selects, so that the vector stays in registers).
+__device__ __forceinline__ uint32_t key_at(const uint4 &v, int j) {
+    const uint32_t word = j < 4 ? (j < 2 ? v.x : v.y) : (j < 6 ? v.z : v.w);
+    return (word >> ((j & 1) * 16)) & 0xffffu;
+}
+
+// The draw over a resident row of 16-bit keys: mass(key) gives an entry's integer mass (0 for an entry that
+// did not survive the filters).  Index order = tile, lane, entry; every sum is an integer sum.
+// With `ties` set, only the first r_cut entries (in index order) equal to tie_key survive, each with mass
+// w_tie; mass() must then return 0 for tie_key.
+// HEAVY = mass() is a long instruction sequence (a polynomial in fp64): the per-entry loops then stay rolled,
+// four entries per iteration for instruction-level parallelism, because 128 inlined copies would not fit the
+// instruction cache.  A cheap mass() (an LDS lookup) is fully unrolled.
+template <bool HEAVY, typename F>
+__device__ __forceinline__ void resident_draw(DenseScalars &ds, const uint4 (&held)[RES_VECS], uint32_t tail_key,
+                                              bool has_tail, int nvec, int tail_index, float u, bool ties,
+                                              uint32_t tie_key, uint32_t r_cut, uint64_t w_tie, F &&mass,
+                                              int64_t *out_slot, float *lp_slot) {
+    const int tid = threadIdx.x;
+    if (tid < 17) {
+        ds.tile_mass[tid] = 0;
+        ds.tile_ties[tid] = 0;
+    }
+    if (tid == 0) ds.hit = -1;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RES_VECS; ++r) {
+        uint64_t w8 = 0;
+        uint32_t t8 = 0;
+        if (tid + r * S_THREADS < nvec) {
+            if constexpr (HEAVY) {
+#pragma unroll 1
+                for (int half = 0; half < 2; ++half) {
+                    const uint32_t lo = half ? held[r].z : held[r].x, hi = half ? held[r].w : held[r].y;
+                    w8 += (mass(lo & 0xffffu) + mass(lo >> 16)) + (mass(hi & 0xffffu) + mass(hi >> 16));
+                }
+            } else {
+                const uint32_t in[4] = {held[r].x, held[r].y, held[r].z, held[r].w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t k0 = in[q] & 0xffffu, k1 = in[q] >> 16;
+                    w8 += mass(k0) + mass(k1);
+                    t8 += ((ties && k0 == tie_key) ? 1u : 0u) + ((ties && k1 == tie_key) ? 1u : 0u);
+                }
+            }
+        }
+        w8 = wave_sum_u64(w8);
+        if ((tid & (kWave - 1)) == 0 && w8 != 0)
+            atomicAdd(reinterpret_cast<unsigned long long *>(&ds.tile_mass[r]), (unsigned long long)w8);
+        if (ties) {
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) t8 += __shfl_xor(t8, off, kWave);
+            if ((tid & (kWave - 1)) == 0 && t8 != 0) atomicAdd(&ds.tile_ties[r], t8);
+        }
+    }
+    {
+        uint64_t wt = has_tail ? mass(tail_key) : 0ull;  // fewer than 8 entries, all in wavefront 0
+        uint32_t tt = (ties && has_tail && tail_key == tie_key) ? 1u : 0u;
+        wt = wave_sum_u64(wt);
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) tt += __shfl_xor(tt, off, kWave);
+        if (tid == 0) {
+            ds.tile_mass[16] = wt;
+            ds.tile_ties[16] = tt;
+        }
+    }
+    __syncthreads();
+    // total per tile = strict mass + the tie-group entries that still fit under r_cut
+    uint64_t z = 0;
+    {
+        uint32_t seen = 0;
+#pragma unroll
+        for (int r = 0; r < 17; ++r) {
+            const uint32_t t = ds.tile_ties[r];
+            const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
+            z += ds.tile_mass[r] + uint64_t(t < room ? t : room) * w_tie;
+            seen += t;
+        }
+    }
+    const uint64_t tau = floor_scale(u, z);
+    uint64_t acc = 0;       // mass before the tile that holds tau
+    uint32_t ties_before = 0;  // tie-group entries before that tile
+    int tile = -1;
+    {
+        uint32_t seen = 0;
+#pragma unroll
+        for (int r = 0; r < 17; ++r) {
+            const uint32_t t = ds.tile_ties[r];
+            const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
+            const uint64_t m = ds.tile_mass[r] + uint64_t(t < room ? t : room) * w_tie;
+            if (tile < 0 && tau < acc + m) { tile = r; ties_before = seen; }
+            if (tile < 0) acc += m;
+            seen += t;
+        }
+    }
+    // held[tile] for a run-time tile, with masks: a chain of selects would be turned into a dynamically
+    // indexed load, and the sixteen vectors would then live in scratch memory instead of registers
+    uint4 cur = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < RES_VECS; ++r) {
+        const uint32_t m = r == tile ? 0xffffffffu : 0u;
+        cur.x |= held[r].x & m;
+        cur.y |= held[r].y & m;
+        cur.z |= held[r].z & m;
+        cur.w |= held[r].w & m;
+    }
+    const bool have = tile >= 0 && tile < 16 && tid + tile * S_THREADS < nvec;
+    if (tile == 16) cur.x = tail_key;  // the tail "tile" holds one entry per lane
+    const int n_here = tile == 16 ? (has_tail ? 1 : 0) : (have ? 8 : 0);
+    uint32_t first_rank = 0;  // index-order rank of this lane's first tie-group entry
+    if (ties) {
+        uint32_t c = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c += (j < n_here && key_at(cur, j) == tie_key) ? 1u : 0u;
+        uint32_t tot;
+        first_rank = ties_before + block_excl_scan<uint32_t>(c, ds.wave_u32, &tot);
+    }
+    // mass of entry j of this lane (the lane's entries are walked twice rather than kept in 16 registers)
+    auto entry_mass = [&](int j, uint32_t &rank) -> uint64_t {
+        if (j >= n_here) return 0ull;
+        const uint32_t k = key_at(cur, j);
+        if (ties && k == tie_key) return (rank++ < r_cut) ? w_tie : 0ull;
+        return mass(k);
+    };
+    uint64_t msum = 0;
+    {
+        uint32_t rank = first_rank;
+#pragma unroll 1
+        for (int j = 0; j < 8; ++j) msum += entry_mass(j, rank);
+    }
+    uint64_t tot;
+    const uint64_t excl = acc + block_excl_scan<uint64_t>(msum, ds.wave_u64, &tot);
+    if (excl <= tau && tau < excl + msum) {
+        uint64_t cum = excl;
+        uint32_t rank = first_rank;
+        const int base = tile == 16 ? tail_index : (tid + tile * S_THREADS) * 8;
+#pragma unroll 1
+        for (int j = 0; j < 8; ++j) {
+            const uint64_t wj = entry_mass(j, rank);
+            cum += wj;
+            if (cum > tau) { ds.hit = base + j; ds.pick_w = wj; break; }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        *out_slot = ds.hit;
+        if (lp_slot != nullptr) *lp_slot = ds.hit >= 0 ? log_ratio(ds.pick_w, z) : __builtin_nanf("");
+    }
+}
+
+// Reads the row into registers as 16-bit keys of the scaled entries; returns the lane's largest key.
+template <typename T, bool HAS_T>
+__device__ __forceinline__ uint32_t resident_load_keys_t(const typename T::raw_t *rp, int vocab, int nvec, float temp,
+                                                         uint4 (&held)[RES_VECS], uint32_t *tail_key,
+                                                         bool *has_tail) {
+    const int tid = threadIdx.x;
+    const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+#pragma unroll
+    for (int r = 0; r < RES_VECS; ++r) {
+        const int v = tid + r * S_THREADS;
+        held[r] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
+    }
+    uint32_t kmax = 0;
+#pragma unroll
+    for (int r = 0; r < RES_VECS; ++r) {
+        if (tid + r * S_THREADS < nvec) {
+            // explicit shifts (no 16-bit pointer accesses): the vectors must stay in registers
+            const uint32_t in[4] = {held[r].x, held[r].y, held[r].z, held[r].w};
+            uint32_t o[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t k0 = elem_key16<T, HAS_T>(in[q] & 0xffffu, temp);
+                const uint32_t k1 = elem_key16<T, HAS_T>(in[q] >> 16, temp);
+                o[q] = k0 | (k1 << 16);
+                kmax = k0 > kmax ? k0 : kmax;
+                kmax = k1 > kmax ? k1 : kmax;
+            }
+            held[r] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    }
+    const int i = nvec * 8 + tid;
+    *has_tail = i < vocab;
+    *tail_key = *has_tail ? elem_key16<T, HAS_T>(uint32_t(rp[i]), temp) : 0u;
+    if (*has_tail) kmax = *tail_key > kmax ? *tail_key : kmax;
+    return kmax;
+}
+template <typename T>
+__device__ __forceinline__ uint32_t resident_load_keys(const typename T::raw_t *rp, int vocab, int nvec, float temp,
+                                                       bool has_t, uint4 (&held)[RES_VECS], uint32_t *tail_key,
+                                                       bool *has_tail) {
+    return has_t ? resident_load_keys_t<T, true>(rp, vocab, nvec, temp, held, tail_key, has_tail)
+                 : resident_load_keys_t<T, false>(rp, vocab, nvec, temp, held, tail_key, has_tail);
+}
+
+template <typename T>
+__device__ __forceinline__ bool resident_ok(int vocab, bool vec) {
+    return vec && T::kBytes == 2 && vocab / 8 <= RES_VECS * S_THREADS;
+}
+
+// No filter at all: every entry survives.
+template <typename T>
+__device__ __forceinline__ bool nofilter_resident(DenseScalars &ds, const typename T::raw_t *rp, int vocab, bool vec,
+                                                  float temp, bool has_t, float u, int64_t *out_slot, float *lp_slot) {
+    if (!resident_ok<T>(vocab, vec)) return false;
+    const int nvec = vocab / 8;
+    uint4 held[RES_VECS];
+    uint32_t tail_key;
+    bool has_tail;
+    const uint32_t lmax = resident_load_keys<T>(rp, vocab, nvec, temp, has_t, held, &tail_key, &has_tail);
+    const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);
+    const float vmax = value_of_key16<T>(kmax);
+    resident_draw<true>(ds, held, tail_key, has_tail, nvec, nvec * 8 + int(threadIdx.x), u, false, 0u, 0xffffffffu, 0ull,
+                  [&](uint32_t k) { return weight_fix(k == kmax ? 0.0f : value_of_key16<T>(k) - vmax); }, out_slot,
+                  lp_slot);
+    return true;
+}
+
+// Word w of the count histogram holds the keys 2w (low half) and 2w + 1 (high half).  A lane later reads
+// 32 consecutive words (128 B) with ds_read_b128; the 16-byte chunk index inside each 128-byte block is
+// XOR-swizzled with the block index so that those reads spread over the banks.
+__device__ __forceinline__ int hist_slot(int word) {
+    return word ^ ((word >> 4) & 0x1c);  // chunk index (bits 2..4) ^= bits 1..3 of the block index (bits 6..8)
+}
+
+template <typename T>
+__device__ __forceinline__ bool dense_resident(unsigned char *lds, const typename T::raw_t *rp, int vocab, bool vec,
+                                               float temp, bool has_t, bool use_k, int top_k, bool use_p, float top_p,
+                                               float u, int64_t *out_slot, float *lp_slot) {
+    if (!resident_ok<T>(vocab, vec)) return false;
+    uint32_t *hist = reinterpret_cast<uint32_t *>(lds);
+    uint32_t *list = hist + D_WORDS;                                   // (key << 16) | count, descending keys
+    uint64_t *table = reinterpret_cast<uint64_t *>(list);              // later: mass of key kcut16 + i
+    DenseScalars &ds = *reinterpret_cast<DenseScalars *>(list + D_LIST_CAP);
+    const int tid = threadIdx.x;
+    const int nvec = vocab / 8;
+
+    // ---- 1. keys into registers, counts into the histogram ------------------------------------------------
+    {
+        uint4 *h4 = reinterpret_cast<uint4 *>(hist);
+        for (int i = tid; i < D_WORDS / 4; i += S_THREADS) h4[i] = make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();
+    uint4 held[RES_VECS];
+    uint32_t tail_key;
+    bool has_tail;
+    const uint32_t lmax = resident_load_keys<T>(rp, vocab, nvec, temp, has_t, held, &tail_key, &has_tail);
+#pragma unroll
+    for (int r = 0; r < RES_VECS; ++r) {
+        if (tid + r * S_THREADS < nvec) {
+            const uint32_t in[4] = {held[r].x, held[r].y, held[r].z, held[r].w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t k0 = in[q] & 0xffffu, k1 = in[q] >> 16;
+                atomicAdd(&hist[hist_slot(k0 >> 1)], (k0 & 1) ? 0x10000u : 1u);
+                atomicAdd(&hist[hist_slot(k1 >> 1)], (k1 & 1) ? 0x10000u : 1u);
+            }
+        }
+    }
+    if (has_tail) atomicAdd(&hist[hist_slot(tail_key >> 1)], (tail_key & 1) ? 0x10000u : 1u);
+    const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);  // its barriers also publish the histogram
+    const float vmax = value_of_key16<T>(kmax);
+
+    // ---- 2. compact the occupied keys, in descending order, into the list ---------------------------------
+    // lane t owns the words [D_WORDS - 32 (t + 1), D_WORDS - 32 t) and walks them from the top
+    const int block = D_WORDS / 32 - 1 - tid;
+    // (the 128 bytes are read twice, 16 at a time, rather than held in 32 registers next to the row)
+    auto chunk_of = [&](int c) {
+        return *reinterpret_cast<const uint4 *>(&hist[(block << 5) | (((c ^ (block >> 1)) & 7) << 2)]);
+    };
+    uint32_t n_occ = 0, n_cnt = 0;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const uint4 wv = chunk_of(c);
+        const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            n_occ += ((q[i] >> 16) != 0) + ((q[i] & 0xffffu) != 0);
+            n_cnt += (q[i] >> 16) + (q[i] & 0xffffu);
+        }
+    }
+    uint32_t occ_total, cnt_total;
+    uint32_t at = block_excl_scan<uint32_t>(n_occ, ds.wave_u32, &occ_total);
+    block_excl_scan<uint32_t>(n_cnt, ds.wave_u32, &cnt_total);
+    // a 16-bit counter that overflowed loses 65,535 or 65,536 entries of the total; more occupied keys than
+    // the list holds: leave the row to the radix path
+    if (cnt_total != uint32_t(vocab) || occ_total > uint32_t(D_LIST_CAP)) return false;
+#pragma unroll
+    for (int c = 7; c >= 0; --c) {
+        const uint4 wv = chunk_of(c);
+        const uint32_t q[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int i = 3; i >= 0; --i) {
+            const uint32_t key_hi = uint32_t(((block << 5) + c * 4 + i) * 2 + 1);
+            if ((q[i] >> 16) != 0) list[at++] = (key_hi << 16) | (q[i] >> 16);
+            if ((q[i] & 0xffffu) != 0) list[at++] = ((key_hi - 1) << 16) | (q[i] & 0xffffu);
+        }
+    }
+    __syncthreads();
+
+    // ---- 3. masses, once per occupied key: lane t takes the entries [t * D_PER_THREAD, ...) ---------------
+    uint32_t ent[D_PER_THREAD];
+    uint64_t wgt[D_PER_THREAD];
+    uint64_t m_local = 0;
+    uint32_t c_local = 0;
+#pragma unroll
+    for (int e = 0; e < D_PER_THREAD; ++e) {
+        const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
+        ent[e] = i < occ_total ? list[i] : 0u;
+        const uint32_t k = ent[e] >> 16, c = ent[e] & 0xffffu;
+        wgt[e] = c ? weight_fix(k == kmax ? 0.0f : value_of_key16<T>(k) - vmax) : 0ull;
+        m_local += wgt[e] * c;
+        c_local += c;
+    }
+    uint64_t z_all;
+    uint32_t c_all;
+    const uint64_t m_before = block_excl_scan<uint64_t>(m_local, ds.wave_u64, &z_all);
+    const uint32_t c_before = block_excl_scan<uint32_t>(c_local, ds.wave_u32, &c_all);
+
+    // ---- 4. top-k: the list entry that holds the top_k-th largest entry; everything down to it survives ----
+    if (tid == 0) {
+        ds.i_topk = occ_total - 1;
+        ds.z_topk = z_all;
+        ds.best_i = -1;
+    }
+    __syncthreads();
+    if (use_k && c_before < uint32_t(top_k) && uint32_t(top_k) <= c_before + c_local) {
+        uint32_t c_run = c_before;
+        uint64_t m_run = m_before;
+#pragma unroll
+        for (int e = 0; e < D_PER_THREAD; ++e) {
+            const uint32_t c = ent[e] & 0xffffu;
+            const bool here = c_run < uint32_t(top_k) && uint32_t(top_k) <= c_run + c;
+            c_run += c;
+            m_run += wgt[e] * c;
+            if (here) {
+                ds.i_topk = uint32_t(tid) * D_PER_THREAD + e;
+                ds.z_topk = m_run;
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t i_topk = ds.i_topk;
+    const uint64_t z_topk = ds.z_topk;
+
+    // ---- 5. top-p: the last entry at or above i_topk whose first element has (mass before it) <= theta -----
+    uint32_t i_cut = i_topk;
+    uint64_t z_kept = z_topk;
+    bool track_ties = false;
+    uint32_t r_cut = 0xffffffffu;
+    uint64_t w_tie = 0;
+    if (use_p) {
+        const uint64_t theta = floor_scale(top_p, z_topk);
+        int best = -1;
+        uint64_t m_run = m_before;
+#pragma unroll
+        for (int e = 0; e < D_PER_THREAD; ++e) {
+            const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
+            const uint32_t c = ent[e] & 0xffffu;
+            if (c != 0 && i <= i_topk && m_run <= theta) best = int(i);
+            m_run += wgt[e] * c;
+        }
+        if (best >= 0) atomicMax(&ds.best_i, best);
+        __syncthreads();
+        i_cut = uint32_t(ds.best_i);
+        if (i_cut / D_PER_THREAD == uint32_t(tid)) {
+            uint64_t m_run2 = m_before;
+#pragma unroll
+            for (int e = 0; e < D_PER_THREAD; ++e) {
+                const uint32_t c = ent[e] & 0xffffu;
+                if (uint32_t(tid) * D_PER_THREAD + e == i_cut) {
+                    ds.before_cut = m_run2;
+                    ds.w_cut = wgt[e];
+                    ds.n_cut = c;
+                }
+                m_run2 += wgt[e] * c;
+            }
+        }
+        __syncthreads();
+        const uint64_t before = ds.before_cut, w_cut = ds.w_cut;
+        const uint64_t n_cut = ds.n_cut;
+        uint64_t r = n_cut;
+        if (w_cut > 0) {
+            const uint64_t fit = (theta - before) / w_cut + 1;  // entries t with before + t * w <= theta
+            r = fit < r ? fit : r;
+        }
+        z_kept = before + r * w_cut;
+        if (r != n_cut) {  // the cut falls inside a tie group: only its first r entries, in index order, survive
+            track_ties = true;
+            r_cut = uint32_t(r);
+            w_tie = w_cut;
+        }
+    }
+    // ---- 6. masses of the surviving keys into a table indexed by key - cut key ------------------------------
+    if (tid == i_cut / D_PER_THREAD) {
+#pragma unroll
+        for (int e = 0; e < D_PER_THREAD; ++e)
+            if (uint32_t(tid) * D_PER_THREAD + e == i_cut) ds.kcut16 = ent[e] >> 16;
+    }
+    __syncthreads();  // also: every lane is done reading the list
+    const uint32_t kcut16 = ds.kcut16;
+    const uint32_t span = kmax - kcut16 + 1;
+    if (span >= uint32_t(D_TABLE_CAP)) return false;
+    for (uint32_t i = tid; i <= span; i += S_THREADS) table[i] = 0;  // table[span] stays 0: the slot of every non-survivor
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < D_PER_THREAD; ++e) {
+        const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
+        if (i <= i_cut && (ent[e] & 0xffffu) != 0) table[(ent[e] >> 16) - kcut16] = wgt[e];
+    }
+    __syncthreads();
+    // ---- 7. draw over the survivors in index order ------------------------------------------------------------
+    (void)z_kept;  // equals the sum of the tile masses below
+    const uint32_t first = track_ties ? kcut16 + 1 : kcut16;  // lowest key whose entries all survive
+    resident_draw<false>(ds, held, tail_key, has_tail, nvec, nvec * 8 + tid, u, track_ties, kcut16, r_cut, w_tie,
+                  [&](uint32_t k) { return table[k >= first ? k - kcut16 : span]; }, out_slot, lp_slot);
+    return true;
+}
+
 // Per-launch parameters.  Each of the three filter parameters is either one value for the whole batch or,
 // when its *_rows pointer is set, one value per row; a row value that is not valid switches that filter
 // off (temperature <= 0 or NaN -> 1, top_k < 0 -> off, top_p outside (0, 1] -> off).
@@ -523,13 +1041,26 @@ struct SampleParams {
 // ---------------------------------------------------------------------------
 // The kernel
 // ---------------------------------------------------------------------------
-template <typename T>
+// DENSE = launched with DENSE_LDS_BYTES of dynamic LDS: the dense-histogram path is available, and the state
+// of the other paths sits at the start of the same memory (the paths never run at the same time).
+template <bool DENSE> __device__ __forceinline__ unsigned char *lds_base() {
+    if constexpr (DENSE) {
+        extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+        return dyn_lds;
+    } else {
+        __shared__ Shared static_lds;
+        return reinterpret_cast<unsigned char *>(&static_lds);
+    }
+}
+
+template <typename T, bool DENSE>
 __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t *__restrict__ logits,
                                                          int vocab, int64_t row_stride, SampleParams prm, int vec,
                                                          int no_fast) {
     constexpr int EPV = T::kPerVec;
     constexpr int LEVELS = Round<T>::kLevels;
-    __shared__ Shared sh;
+    unsigned char *const lds = lds_base<DENSE>();
+    Shared &sh = *reinterpret_cast<Shared *>(lds);
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.x;
     const typename T::raw_t *rp = logits + row * row_stride;
@@ -553,6 +1084,17 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (use_k && top_k <= S_THREADS && !no_fast) {
         if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot)) return;
         __syncthreads();
+    } else if (!use_k && !use_p && !no_fast) {
+        if constexpr (T::kBytes == 2) {
+            if (nofilter_resident<T>(sh.ds, rp, vocab, vec, temp, has_t, u, out + row, lp_slot)) return;
+            __syncthreads();
+        }
+    } else if (!no_fast) {
+        if constexpr (DENSE && T::kBytes == 2) {
+            if (dense_resident<T>(lds, rp, vocab, vec, temp, has_t, use_k, top_k, use_p, top_p, u, out + row, lp_slot))
+                return;
+            __syncthreads();
+        }
     }
 
     // ---- pass 0: row maximum and the level-0 count histogram --------------------------
@@ -736,6 +1278,11 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     }
 }
 
+__global__ __launch_bounds__(256) void mass_fixed_kernel(const float *__restrict__ d, int64_t n, uint64_t *__restrict__ out) {
+    const int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = weight_fix(d[i]);
+}
+
 // KA_SAMPLE_RADIX_ONLY=1 switches the top-k fast path off (the tests use it to run both paths on every case).
 inline bool force_radix_path() {
     const char *e = getenv("KA_SAMPLE_RADIX_ONLY");
@@ -764,10 +1311,29 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
         return fail(KA_ERR_WORKSPACE, "sample: workspace of %zu B, need %zu B", workspace_bytes,
                     ka_sample_workspace_bytes(batch, vocab));
     const bool aligned = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * T::kBytes) % 16 == 0);
-    hipLaunchKernelGGL((sample_rows<T>), dim3(unsigned(batch)), dim3(S_THREADS), 0,
-                       static_cast<hipStream_t>(hip_stream),
-                       static_cast<const typename T::raw_t *>(logits), int(vocab), row_stride, prm,
-                       aligned ? 1 : 0, force_radix_path() ? 1 : 0);
+    const bool no_fast = force_radix_path();
+    // The dense-histogram path needs 157 KB of LDS (one workgroup per CU).  It serves top-p without top-k and
+    // top_k > 1024 on 16-bit rows that fit in registers; with per-row parameters any row may need it.
+    bool dense = false;
+    if (T::kBytes == 2 && aligned && !no_fast && vocab / 8 <= RES_VECS * S_THREADS) {
+        const bool per_row = prm.top_k_rows != nullptr || prm.top_p_rows != nullptr;
+        const bool k_on = prm.top_k > 0 && prm.top_k < vocab;
+        dense = per_row || (k_on && prm.top_k > S_THREADS) || (!k_on && prm.top_p < 1.0f);
+    }
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const typename T::raw_t *lp = static_cast<const typename T::raw_t *>(logits);
+    if constexpr (T::kBytes == 2) {
+      if (dense) {
+        const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(sample_rows<T, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, int(DENSE_LDS_BYTES));
+        if (rc != hipSuccess) return check_hip(rc, "sample: reserving LDS for the dense-histogram path");
+        hipLaunchKernelGGL((sample_rows<T, true>), dim3(unsigned(batch)), dim3(S_THREADS), DENSE_LDS_BYTES, stream, lp,
+                           int(vocab), row_stride, prm, aligned ? 1 : 0, 0);
+        return check_hip(hipGetLastError(), "sample launch");
+      }
+    }
+    hipLaunchKernelGGL((sample_rows<T, false>), dim3(unsigned(batch)), dim3(S_THREADS), 0, stream, lp, int(vocab),
+                       row_stride, prm, aligned ? 1 : 0, no_fast ? 1 : 0);
     return check_hip(hipGetLastError(), "sample launch");
 }
 
@@ -825,6 +1391,17 @@ KA_EXPORT int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t
     return ka::launch<ka::F32>(logits, batch, vocab, row_stride,
                               ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids), workspace,
                               workspace_bytes, hip_stream);
+}
+
+KA_EXPORT int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, void *hip_stream) {
+    using namespace ka;
+    if (n < 0) return fail(KA_ERR_BAD_ARG, "mass: n %lld < 0", (long long)n);
+    if (n == 0) return KA_OK;
+    if (d == nullptr || out == nullptr) return fail(KA_ERR_BAD_ARG, "mass: null pointer argument");
+    if ((n + 255) / 256 >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "mass: n too large");
+    hipLaunchKernelGGL(mass_fixed_kernel, dim3(unsigned((n + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream), d, n, out);
+    return check_hip(hipGetLastError(), "mass launch");
 }
 
 KA_EXPORT int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,

@@ -29,6 +29,8 @@ def lib() -> ctypes.CDLL:
         handle = ctypes.CDLL(str(path))
         handle.ka_oracle_weight.restype = c_uint64
         handle.ka_oracle_weight.argtypes = [c_float]
+        handle.ka_oracle_weight_libm.restype = c_uint64
+        handle.ka_oracle_weight_libm.argtypes = [c_float]
         handle.ka_oracle_floor_scale.restype = c_uint64
         handle.ka_oracle_floor_scale.argtypes = [c_float, c_uint64]
         handle.ka_oracle_scale.restype = None
@@ -43,6 +45,11 @@ def lib() -> ctypes.CDLL:
 def weight(d: float) -> int:
     """W(d) = trunc(2^40 * exp(d)) as the oracle evaluates it."""
     return int(lib().ka_oracle_weight(d))
+
+
+def weight_libm(d: float) -> int:
+    """The same function built on libm's fma() instead of the hardware instruction."""
+    return int(lib().ka_oracle_weight_libm(d))
 
 
 def floor_scale(s: float, z: int) -> int:

@@ -118,32 +118,41 @@ static uint32_t key_of(float y) {
 /*
  * W(d) = trunc(2^40 * exp(d)) for d <= 0, by a fixed sequence of IEEE double operations:
  *   t = d * log2(e);  n = trunc(t - 0.5);  f = t - n  (|f| <= 0.5);  g = f * ln 2;
- *   p = sum_{k=0..11} g^k / k!  (Horner, separate multiply and add);  W = trunc(p * 2^(40+n)).
+ *   p = sum_{k=0..11} g^k / k!  (Horner with fma(), one rounding per step);  W = trunc(p * 2^(40+n)).
  * W(0) = 2^40 exactly; W(d) = 0 once t < -41.
  */
-uint64_t ka_oracle_weight(float d) {
-    /* 1/k! rounded to nearest double, k = 0..11 */
-    static const double C[12] = {0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,
-                                 0x1.5555555555555p-3,  0x1.5555555555555p-5,  0x1.1111111111111p-7,
-                                 0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16,
-                                 0x1.71de3a556c734p-19, 0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26};
-    const double LOG2E = 0x1.71547652b82fep+0, LN2 = 0x1.62e42fefa39efp-1;
-    if (!(d <= 0.0f)) return d > 0.0f ? (uint64_t)1 << KA_FIX_BITS : 0; /* d > 0 cannot occur; NaN -> 0 */
-    double t = (double)d * LOG2E;
-    if (t < -41.0) return 0;
-    int n = (int)(t - 0.5);
-    double f = t - (double)n;
-    double g = f * LN2;
-    double p = C[11];
-    for (int k = 10; k >= 0; --k) {
-        p = p * g;
-        p = p + C[k];
-    }
-    uint64_t pow2_bits = (uint64_t)(1023 + KA_FIX_BITS + n) << 52;
-    double scale;
-    memcpy(&scale, &pow2_bits, 8);
+/* One body, compiled twice: with the hardware fused multiply-add where the CPU has one, and with libm's
+ * fma() (exact by C99) elsewhere.  Both round each Horner step once, so they return the same integers. */
+#define KA_WEIGHT_BODY(FMA)                                                                               \
+    static const double C[12] = {0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,      \
+                                 0x1.5555555555555p-3,  0x1.5555555555555p-5,  0x1.1111111111111p-7,      \
+                                 0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16,     \
+                                 0x1.71de3a556c734p-19, 0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26};    \
+    const double LOG2E = 0x1.71547652b82fep+0, LN2 = 0x1.62e42fefa39efp-1;                                \
+    if (!(d <= 0.0f)) return d > 0.0f ? (uint64_t)1 << KA_FIX_BITS : 0; /* d > 0 cannot occur; NaN -> 0 */ \
+    double t = (double)d * LOG2E;                                                                         \
+    if (t < -41.0) return 0;                                                                              \
+    int n = (int)(t - 0.5);                                                                               \
+    double f = t - (double)n;                                                                             \
+    double g = f * LN2;                                                                                   \
+    double p = C[11];                                                                                     \
+    for (int k = 10; k >= 0; --k) p = FMA(p, g, C[k]);                                                    \
+    uint64_t pow2_bits = (uint64_t)(1023 + KA_FIX_BITS + n) << 52;                                        \
+    double scale;                                                                                         \
+    memcpy(&scale, &pow2_bits, 8);                                                                        \
     return (uint64_t)(p * scale);
+
+__attribute__((target("fma"))) static uint64_t weight_hw(float d) { KA_WEIGHT_BODY(__builtin_fma) }
+static uint64_t weight_sw(float d) { KA_WEIGHT_BODY(fma) }
+
+uint64_t ka_oracle_weight(float d) {
+    static int have_fma = -1;
+    if (have_fma < 0) have_fma = __builtin_cpu_supports("fma") ? 1 : 0;
+    return have_fma ? weight_hw(d) : weight_sw(d);
 }
+
+/* The libm-fma() build of the same function, exported for the test that compares the two. */
+uint64_t ka_oracle_weight_libm(float d) { return weight_sw(d); }
 
 /* floor(s * z) for an fp32 scalar 0 <= s < 1 and an integer z < 2^62, exactly. */
 static uint64_t floor_scale(float s, uint64_t z) {

@@ -36,6 +36,12 @@ def test_weight_is_floor_of_scaled_exp():
     assert all(a >= b for a, b in zip(ws, ws[1:]))          # monotone
 
 
+def test_weight_does_not_depend_on_how_fma_is_provided():
+    g = torch.Generator().manual_seed(3)
+    for d in (-torch.rand(3000, generator=g) * 30).tolist() + [0.0, -1e-30, -28.4, -28.5]:
+        assert exact.weight(f32(d)) == exact.weight_libm(f32(d))
+
+
 def test_floor_scale_is_exact():
     g = torch.Generator().manual_seed(1)
     for s in torch.rand(300, generator=g).tolist() + [0.0, 2.0 ** -149, 2.0 ** -126, 1 - 2.0 ** -24, 0.9, 0.5]:

@@ -246,3 +246,22 @@ def test_nan_and_infinite_logits_on_both_paths(sampler, dtype, monkeypatch):
             got = run(sampler, logits, uu, k, p, temp)
             assert torch.equal(got, want), f"radix_only={radix_only} k={k} p={p} T={temp}"
         monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
+
+
+def test_mass_function_is_bit_exact_against_the_oracle(sampler):
+    """W(d) on the GPU (ka_sample_mass_fixed) against oracle/ka_oracle.c for 200k random d in (-31, 0], every
+    d = -i/256, and the special values: the integers every sampled id is built from must be identical."""
+    import ctypes
+    g = torch.Generator().manual_seed(77)
+    d = torch.cat([-torch.rand(200000, generator=g) * 31, -torch.arange(0, 8192) / 256.0,
+                   torch.tensor([0.0, -0.0, -1e-38, -1e-8, -28.4, -28.42, -28.5, -40.0, -88.0, -1e30, -math.inf,
+                                 math.nan, 1.0])]).float()
+    dd = d.cuda()
+    out = torch.empty(d.numel(), dtype=torch.int64, device="cuda")
+    lib = sampler._lib
+    rc = lib.ka_sample_mass_fixed(dd.data_ptr(), d.numel(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    got = out.cpu().tolist()
+    want = [exact.weight(x) for x in d.tolist()]
+    bad = [(x, a, b) for x, a, b in zip(d.tolist(), got, want) if a != b]
+    assert not bad, bad[:5]
