@@ -265,3 +265,30 @@ def test_mass_function_is_bit_exact_against_the_oracle(sampler):
     want = [exact.weight(x) for x in d.tolist()]
     bad = [(x, a, b) for x, a, b in zip(d.tolist(), got, want) if a != b]
     assert not bad, bad[:5]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_randomised_shapes_modes_and_value_grids(sampler, seed):
+    """A sweep over the paths behind `sample`: random vocabulary sizes (ragged tails, tiny rows, rows of one
+    tile, rows longer than the register-resident limit), value grids from continuous to heavily tied, all
+    three dtypes, every filter combination.  Every id must equal the exact oracle's."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    vocabs = [1, 7, 8, 9, 1023, 1024, 8191, 8192, 8200, 40000, 65537, 128256, 131072, 131080, 140001]
+    for trial in range(10):
+        vocab = vocabs[int(torch.randint(0, len(vocabs), (1,), generator=g))]
+        dtype = DTYPES[int(torch.randint(0, 3, (1,), generator=g))]
+        rows = 6
+        spread = float(torch.rand(1, generator=g)) * 6 + 0.2
+        logits = torch.randn(rows, vocab, generator=g) * spread
+        grid = [0.0, 0.0, 0.25, 1.0, 4.0][int(torch.randint(0, 5, (1,), generator=g))]
+        if grid:
+            logits = (logits / grid).round() * grid                     # ties: few distinct values
+        logits = logits.to(dtype)
+        k = [None, None, 1, 5, 50, 1024, 1025, 3000, vocab, vocab + 5][int(torch.randint(0, 10, (1,), generator=g))]
+        p = [None, None, 0.05, 0.5, 0.9, 0.999, 1.0][int(torch.randint(0, 7, (1,), generator=g))]
+        temp = [1.0, 1.0, 0.7, 1.3, 0.05, 25.0][int(torch.randint(0, 6, (1,), generator=g))]
+        u = torch.rand(rows, generator=g)
+        got = run(sampler, logits, u, k, p, temp)
+        want = exact.sample(logits, temp, k, p, u)
+        assert torch.equal(got, want), (f"trial {trial}: vocab={vocab} dtype={dtype} grid={grid} spread={spread:.2f} "
+                                        f"k={k} p={p} T={temp}: rows {(got != want).nonzero().flatten().tolist()}")
