@@ -94,6 +94,21 @@ int ka_logprob_backward_f32(const void *logits, int64_t n_rows, int64_t vocab, i
                             int64_t dlogits_stride, void *hip_stream);
 
 /*
+ * GRPO per-token objective from log-probabilities (all arrays fp32 [n], n = G * L tokens):
+ *     ratio = exp(logp_new - logp_old)            (logp_old null: ratio = 1, the on-policy case)
+ *     surr  = min(ratio * A, clamp(ratio, 1 - clip_low, 1 + clip_high) * A)
+ *     kl    = exp(logp_ref - logp_new) - (logp_ref - logp_new) - 1      (logp_ref null: 0)
+ *     out_loss  = -(surr - beta * kl)
+ *     out_dlogp = d out_loss / d logp_new   (feeds ka_logprob_backward_* as `grad`)
+ * Each output pointer may be null.  No counterpart in the reference, which stops at the log-probabilities
+ * (rl_engine/kernels/sampling.py:92-112) and names the advantage step only in README.md:49; this is the
+ * elementwise epilogue a GRPO trainer applies to them.
+ */
+int ka_grpo_token_terms(const float *logp_new, const float *logp_old, const float *logp_ref,
+                        const float *advantages, int64_t n, float clip_low, float clip_high, float beta,
+                        float *out_loss, float *out_kl, float *out_dlogp, void *hip_stream);
+
+/*
  * Fused temperature -> top-k -> top-p -> draw, one token id per row.
  * Replaces SamplerBackend.sample (rl_engine/kernels/sampling.py:39-88) with the
  * filter semantics of native_sampling (benchmarks/benchmark_sampling.py:12-37):

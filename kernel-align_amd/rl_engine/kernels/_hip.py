@@ -37,6 +37,8 @@ SIGNATURES = {
     "ka_logprob_backward_bf16": (c_int, _BACKWARD_ARGS),
     "ka_logprob_backward_f16": (c_int, _BACKWARD_ARGS),
     "ka_logprob_backward_f32": (c_int, _BACKWARD_ARGS),
+    "ka_grpo_token_terms": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_float, c_float, c_float,
+                                    c_void_p, c_void_p, c_void_p, c_void_p]),
     "ka_sample_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "ka_sample_topk_topp_bf16": (c_int, _SAMPLE_ARGS),
     "ka_sample_topk_topp_f16": (c_int, _SAMPLE_ARGS),

@@ -174,6 +174,49 @@ class SamplerBackend(nn.Module):
                 _hip.check(status, fn_name)
         return logits if inplace else out_rows.view(logits.shape)
 
+    @torch.inference_mode()
+    def grpo_token_loss(self, logp_new, advantages, logp_old=None, logp_ref=None, clip_low=0.2, clip_high=0.2,
+                        beta=0.0):
+        """Per-token GRPO terms from log-probabilities: ``(loss, kl, dloss_dlogp)``, each fp32 of logp_new's shape.
+
+        ``ratio = exp(logp_new - logp_old)`` (1 when ``logp_old`` is None), clipped surrogate with
+        ``advantages`` (same shape, or [G] / [G, 1] for one advantage per sequence of a [G, L] batch), k3 KL
+        estimate to ``logp_ref`` weighted by ``beta``.  ``dloss_dlogp`` is what ``compute_logp_backward`` takes
+        as ``grad_logp``.
+        """
+        _require_gpu(logp_new, "logp_new")
+        shape = tuple(logp_new.shape)
+
+        def flat(t, name):
+            if t is None:
+                return None
+            if tuple(t.shape) != shape:
+                raise ValueError(f"{name} shape {tuple(t.shape)} != logp_new shape {shape}")
+            return t.to(device=logp_new.device, dtype=torch.float32).contiguous().view(-1)
+
+        adv = advantages
+        if adv.dim() >= 1 and adv.dim() <= len(shape) and tuple(adv.shape) != shape:
+            if adv.dim() == 1 and len(shape) == 2 and adv.shape[0] == shape[0]:
+                adv = adv.unsqueeze(-1)
+            try:
+                adv = adv.expand(shape)
+            except RuntimeError:
+                raise ValueError(f"advantages shape {tuple(advantages.shape)} does not broadcast to {shape}") from None
+        new, old, ref, adv = flat(logp_new, "logp_new"), flat(logp_old, "logp_old"), flat(logp_ref, "logp_ref"), \
+            flat(adv, "advantages")
+        n = new.numel()
+        loss = torch.empty(n, dtype=torch.float32, device=new.device)
+        kl = torch.empty_like(loss)
+        dlogp = torch.empty_like(loss)
+        with torch.cuda.device(new.device):
+            status = self._lib.ka_grpo_token_terms(
+                new.data_ptr(), old.data_ptr() if old is not None else None,
+                ref.data_ptr() if ref is not None else None, adv.data_ptr(), n, float(clip_low), float(clip_high),
+                float(beta), loss.data_ptr(), kl.data_ptr(), dlogp.data_ptr(),
+                torch.cuda.current_stream().cuda_stream)
+        _hip.check(status, "ka_grpo_token_terms")
+        return loss.view(shape), kl.view(shape), dlogp.view(shape)
+
     # ----------------------------------------------------------------- sampling
     @torch.inference_mode()
     def sample(self, logits, top_k=None, top_p=None, temperature=1.0, deterministic=True,
