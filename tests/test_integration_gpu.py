@@ -18,20 +18,26 @@ def test_hip_graph_replays_match_eager(sampler):
     weight = (torch.randn(5000, 256, generator=g, device="cuda") * 0.1).bfloat16()
     hid = torch.randint(0, 5000, (300,), generator=g, device="cuda")
     eager = (sampler.compute_logp(logits, ids), sampler.sample(slog, top_k=50, top_p=0.9, temperature=0.7, uniforms=u),
-             sampler.fused_linear_logp(hidden, weight, hid))
+             sampler.fused_linear_logp(hidden, weight, hid),
+             sampler.sample(slog, top_p=0.9, temperature=0.7, uniforms=u),      # dense-histogram path (157 KB of LDS)
+             sampler.sample(slog, uniforms=u))                                   # no filter
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         lp = sampler.compute_logp(logits, ids)
         tok = sampler.sample(slog, top_k=50, top_p=0.9, temperature=0.7, uniforms=u)
         fl = sampler.fused_linear_logp(hidden, weight, hid)
+        tok_p = sampler.sample(slog, top_p=0.9, temperature=0.7, uniforms=u)
+        tok_all = sampler.sample(slog, uniforms=u)
     for replay in range(3):
         with torch.inference_mode():  # the operators return inference tensors, as the reference's do
-            lp.zero_(); tok.zero_(); fl.zero_()
+            lp.zero_(); tok.zero_(); fl.zero_(); tok_p.zero_(); tok_all.zero_()
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(lp, eager[0]) and torch.equal(tok, eager[1]) and torch.equal(fl, eager[2]), replay
+        assert torch.equal(tok_p, eager[3]) and torch.equal(tok_all, eager[4]), replay
+        assert torch.equal(tok_p.cpu(), exact.sample(slog.cpu(), 0.7, None, 0.9, u.cpu()))
         # eager work between replays
         assert torch.equal(sampler.compute_logp(logits, ids), eager[0])
 
