@@ -152,8 +152,8 @@ struct Candidates {            // 24 KB, same footprint as the histograms
 struct DenseScalars {
     uint64_t wave_u64[S_WAVES];
     uint32_t wave_u32[S_WAVES];
-    uint64_t tile_mass[17];  // 16 tiles of 8192 entries + the ragged tail
-    uint32_t tile_ties[17];  // entries equal to the cut key in each tile
+    uint64_t seg_mass[S_WAVES + 1];  // dense path: mass of each wavefront's share of the row, and of the ragged tail
+    uint32_t seg_ties[S_WAVES + 1];  // ... and its number of tie-group entries
     uint64_t z_topk, before_cut, w_cut, pick_w;
     uint32_t i_topk, n_cut, kcut16;
     int best_i;
@@ -528,8 +528,9 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
 // order-preserving key of its scaled value, so the later passes neither touch memory nor divide again.
 // Since a 16-bit dtype has only 65,536 values, an entry's integer mass is a function of its key.
 //
-//   no filter   : one pass evaluates every entry's mass and leaves the mass of each 8192-entry tile in LDS;
-//                 the draw walks tile totals, then the per-lane sums of one tile, then eight entries.
+//   no filter   : one pass evaluates every entry's mass; each lane owns a contiguous run of entries, so one
+//                 block-wide prefix sum of the lane totals finds the lane that holds the draw, which then
+//                 finds the vector and the entry.
 //   dense path  : (top-p without top-k, or top_k > 1024) a count histogram over all 65,536 keys in LDS
 //                 (16-bit counters, two per word) is compacted into a list of the occupied keys in
 //                 descending order; masses are evaluated once per occupied key (a few thousand instead of
@@ -604,149 +605,149 @@ __device__ __forceinline__ uint32_t block_max_u32_buf(uint32_t v, uint32_t *wave
     return r;
 }
 
-// Entry j (0..7) of a vector of eight 16-bit keys, for a j that is not a compile-time constant (register
-// selects, so that the vector stays in registers).
-__device__ __forceinline__ uint32_t key_at(const uint4 &v, int j) {
-    const uint32_t word = j < 4 ? (j < 2 ? v.x : v.y) : (j < 6 ? v.z : v.w);
-    return (word >> ((j & 1) * 16)) & 0xffffu;
+// Layout of a resident row: lane t owns the vectors [t * vpl, (t + 1) * vpl) (vpl = ceil(nvec / 1024) <= 16),
+// a contiguous run of entries, so index order is (lane, vector, entry) and one block-wide prefix sum over
+// per-lane totals finds the lane that holds the draw.  (The loads are 16 bytes per lane at a stride of
+// 16 * vpl bytes; the lines are shared by the lane's consecutive loads and come from L1 / L2.)
+__device__ __forceinline__ bool lane_has_vec(int r, int vpl, int nvec) {
+    return r < vpl && int(threadIdx.x) * vpl + r < nvec;
 }
 
 // The draw over a resident row of 16-bit keys: mass(key) gives an entry's integer mass (0 for an entry that
-// did not survive the filters).  Index order = tile, lane, entry; every sum is an integer sum.
+// did not survive the filters); every sum is an integer sum.
 // With `ties` set, only the first r_cut entries (in index order) equal to tie_key survive, each with mass
 // w_tie; mass() must then return 0 for tie_key.
 // HEAVY = mass() is a long instruction sequence (a polynomial in fp64): the per-entry loops then stay rolled,
 // four entries per iteration for instruction-level parallelism, because 128 inlined copies would not fit the
 // instruction cache.  A cheap mass() (an LDS lookup) is fully unrolled.
 template <bool HEAVY, typename F>
-__device__ __forceinline__ void resident_draw(DenseScalars &ds, const uint4 (&held)[RES_VECS], uint32_t tail_key,
-                                              bool has_tail, int nvec, int tail_index, float u, bool ties,
-                                              uint32_t tie_key, uint32_t r_cut, uint64_t w_tie, F &&mass,
-                                              int64_t *out_slot, float *lp_slot) {
+__device__ __forceinline__ void resident_draw(DenseScalars &ds, const uint4 (&held)[RES_VECS], int vpl, int nvec,
+                                              uint32_t tail_key, bool has_tail, int tail_index, bool any_tail,
+                                              float u, bool ties, uint32_t tie_key, uint32_t r_cut, uint64_t w_tie,
+                                              F &&mass, int64_t *out_slot, float *lp_slot) {
     const int tid = threadIdx.x;
-    if (tid < 17) {
-        ds.tile_mass[tid] = 0;
-        ds.tile_ties[tid] = 0;
-    }
     if (tid == 0) ds.hit = -1;
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < RES_VECS; ++r) {
+    // mass of one vector without its tie-group entries, and the number of those
+    auto vec_mass = [&](const uint4 &v) -> uint64_t {
         uint64_t w8 = 0;
-        uint32_t t8 = 0;
-        if (tid + r * S_THREADS < nvec) {
-            if constexpr (HEAVY) {
+        if constexpr (HEAVY) {
 #pragma unroll 1
-                for (int half = 0; half < 2; ++half) {
-                    const uint32_t lo = half ? held[r].z : held[r].x, hi = half ? held[r].w : held[r].y;
-                    w8 += (mass(lo & 0xffffu) + mass(lo >> 16)) + (mass(hi & 0xffffu) + mass(hi >> 16));
-                }
-            } else {
-                const uint32_t in[4] = {held[r].x, held[r].y, held[r].z, held[r].w};
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint32_t k0 = in[q] & 0xffffu, k1 = in[q] >> 16;
-                    w8 += mass(k0) + mass(k1);
-                    t8 += ((ties && k0 == tie_key) ? 1u : 0u) + ((ties && k1 == tie_key) ? 1u : 0u);
-                }
+            for (int half = 0; half < 2; ++half) {
+                const uint32_t lo = half ? v.z : v.x, hi = half ? v.w : v.y;
+                w8 += (mass(lo & 0xffffu) + mass(lo >> 16)) + (mass(hi & 0xffffu) + mass(hi >> 16));
             }
-        }
-        w8 = wave_sum_u64(w8);
-        if ((tid & (kWave - 1)) == 0 && w8 != 0)
-            atomicAdd(reinterpret_cast<unsigned long long *>(&ds.tile_mass[r]), (unsigned long long)w8);
-        if (ties) {
+        } else {
+            const uint32_t in[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) t8 += __shfl_xor(t8, off, kWave);
-            if ((tid & (kWave - 1)) == 0 && t8 != 0) atomicAdd(&ds.tile_ties[r], t8);
+            for (int q = 0; q < 4; ++q) w8 += mass(in[q] & 0xffffu) + mass(in[q] >> 16);
         }
-    }
-    {
-        uint64_t wt = has_tail ? mass(tail_key) : 0ull;  // fewer than 8 entries, all in wavefront 0
-        uint32_t tt = (ties && has_tail && tail_key == tie_key) ? 1u : 0u;
-        wt = wave_sum_u64(wt);
+        return w8;
+    };
+    auto vec_ties = [&](const uint4 &v) -> uint32_t {
+        const uint32_t in[4] = {v.x, v.y, v.z, v.w};
+        uint32_t t = 0;
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) tt += __shfl_xor(tt, off, kWave);
-        if (tid == 0) {
-            ds.tile_mass[16] = wt;
-            ds.tile_ties[16] = tt;
-        }
-    }
-    __syncthreads();
-    // total per tile = strict mass + the tie-group entries that still fit under r_cut
-    uint64_t z = 0;
-    {
-        uint32_t seen = 0;
-#pragma unroll
-        for (int r = 0; r < 17; ++r) {
-            const uint32_t t = ds.tile_ties[r];
-            const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
-            z += ds.tile_mass[r] + uint64_t(t < room ? t : room) * w_tie;
-            seen += t;
-        }
-    }
-    const uint64_t tau = floor_scale(u, z);
-    uint64_t acc = 0;       // mass before the tile that holds tau
-    uint32_t ties_before = 0;  // tie-group entries before that tile
-    int tile = -1;
-    {
-        uint32_t seen = 0;
-#pragma unroll
-        for (int r = 0; r < 17; ++r) {
-            const uint32_t t = ds.tile_ties[r];
-            const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
-            const uint64_t m = ds.tile_mass[r] + uint64_t(t < room ? t : room) * w_tie;
-            if (tile < 0 && tau < acc + m) { tile = r; ties_before = seen; }
-            if (tile < 0) acc += m;
-            seen += t;
-        }
-    }
-    // held[tile] for a run-time tile, with masks: a chain of selects would be turned into a dynamically
-    // indexed load, and the sixteen vectors would then live in scratch memory instead of registers
-    uint4 cur = make_uint4(0, 0, 0, 0);
+        for (int q = 0; q < 4; ++q) t += (((in[q] & 0xffffu) == tie_key) ? 1u : 0u) + (((in[q] >> 16) == tie_key) ? 1u : 0u);
+        return ties ? t : 0u;
+    };
+    // ---- masses of this lane in four groups of four vectors, tie-group entries of the lane ---------------------
+    uint64_t gsum[4] = {0, 0, 0, 0};
+    uint32_t lane_ties = 0;
 #pragma unroll
     for (int r = 0; r < RES_VECS; ++r) {
-        const uint32_t m = r == tile ? 0xffffffffu : 0u;
-        cur.x |= held[r].x & m;
-        cur.y |= held[r].y & m;
-        cur.z |= held[r].z & m;
-        cur.w |= held[r].w & m;
+        if (lane_has_vec(r, vpl, nvec)) {
+            gsum[r >> 2] += vec_mass(held[r]);
+            lane_ties += vec_ties(held[r]);
+        }
     }
-    const bool have = tile >= 0 && tile < 16 && tid + tile * S_THREADS < nvec;
-    if (tile == 16) cur.x = tail_key;  // the tail "tile" holds one entry per lane
-    const int n_here = tile == 16 ? (has_tail ? 1 : 0) : (have ? 8 : 0);
-    uint32_t first_rank = 0;  // index-order rank of this lane's first tie-group entry
-    if (ties) {
-        uint32_t c = 0;
+    // ---- lane totals in index order ----------------------------------------------------------------------------
+    uint32_t first_rank = 0, all_vec_ties = 0;  // rank of the lane's first tie-group entry; such entries in all vectors
+    if (ties) first_rank = block_excl_scan<uint32_t>(lane_ties, ds.wave_u32, &all_vec_ties);
+    const uint32_t lane_room = first_rank < r_cut ? r_cut - first_rank : 0u;
+    const uint64_t lane_total = (gsum[0] + gsum[1]) + (gsum[2] + gsum[3]) +
+                                uint64_t(lane_ties < lane_room ? lane_ties : lane_room) * w_tie;
+    uint64_t z_vec;
+    const uint64_t lane_before = block_excl_scan<uint64_t>(lane_total, ds.wave_u64, &z_vec);
+    // the ragged tail of the row (fewer than 8 entries after the last vector, one per lane of wavefront 0)
+    uint64_t tail_mass = 0, tail_before = 0, z_tail = 0;
+    if (any_tail) {
+        uint32_t tail_rank = 0, tot_t;
+        const bool tail_tie = ties && has_tail && tail_key == tie_key;
+        if (ties) tail_rank = all_vec_ties + block_excl_scan<uint32_t>(tail_tie ? 1u : 0u, ds.wave_u32, &tot_t);
+        if (has_tail) tail_mass = tail_tie ? (tail_rank < r_cut ? w_tie : 0ull) : mass(tail_key);
+        tail_before = z_vec + block_excl_scan<uint64_t>(tail_mass, ds.wave_u64, &z_tail);
+    }
+    const uint64_t z = z_vec + z_tail;
+    const uint64_t tau = floor_scale(u, z);
+    // ---- the lane that holds tau finds the group, the vector, the entry ------------------------------------------
+    // (vectors are picked with masks: a chain of selects on a run-time index would be turned into a dynamically
+    // indexed load and move the sixteen vectors to scratch memory)
+    if (lane_before <= tau && tau < lane_before + lane_total) {
+        uint64_t cum = lane_before;
+        uint32_t rank = first_rank;
+        uint4 c4[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c += (j < n_here && key_at(cur, j) == tie_key) ? 1u : 0u;
-        uint32_t tot;
-        first_rank = ties_before + block_excl_scan<uint32_t>(c, ds.wave_u32, &tot);
-    }
-    // mass of entry j of this lane (the lane's entries are walked twice rather than kept in 16 registers)
-    auto entry_mass = [&](int j, uint32_t &rank) -> uint64_t {
-        if (j >= n_here) return 0ull;
-        const uint32_t k = key_at(cur, j);
-        if (ties && k == tie_key) return (rank++ < r_cut) ? w_tie : 0ull;
-        return mass(k);
-    };
-    uint64_t msum = 0;
-    {
-        uint32_t rank = first_rank;
-#pragma unroll 1
-        for (int j = 0; j < 8; ++j) msum += entry_mass(j, rank);
-    }
-    uint64_t tot;
-    const uint64_t excl = acc + block_excl_scan<uint64_t>(msum, ds.wave_u64, &tot);
-    if (excl <= tau && tau < excl + msum) {
-        uint64_t cum = excl;
-        uint32_t rank = first_rank;
-        const int base = tile == 16 ? tail_index : (tid + tile * S_THREADS) * 8;
+        for (int i = 0; i < 4; ++i) c4[i] = make_uint4(0, 0, 0, 0);
+        int g_hit = -1;
+        uint64_t cum_g = 0;
+        uint32_t rank_g = 0;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            uint32_t tg = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (lane_has_vec(g * 4 + i, vpl, nvec)) tg += vec_ties(held[g * 4 + i]);
+            const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
+            const uint64_t gt = gsum[g] + uint64_t(tg < room ? tg : room) * w_tie;
+            const bool here = g_hit < 0 && tau < cum + gt;
+            const uint32_t m = here ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                c4[i].x |= held[g * 4 + i].x & m;
+                c4[i].y |= held[g * 4 + i].y & m;
+                c4[i].z |= held[g * 4 + i].z & m;
+                c4[i].w |= held[g * 4 + i].w & m;
+            }
+            if (here) { g_hit = g; cum_g = cum; rank_g = rank; }
+            cum += gt;
+            rank += tg;
+        }
+        uint4 cur = make_uint4(0, 0, 0, 0);
+        int r_hit = -1;
+        uint64_t cum_v = 0;
+        uint32_t rank_v = 0;
+        cum = cum_g;
+        rank = rank_g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool present = lane_has_vec(g_hit * 4 + i, vpl, nvec);
+            const uint32_t tv = present ? vec_ties(c4[i]) : 0u;
+            const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
+            const uint64_t vt = (present ? vec_mass(c4[i]) : 0ull) + uint64_t(tv < room ? tv : room) * w_tie;
+            const bool here = r_hit < 0 && tau < cum + vt;
+            const uint32_t m = here ? 0xffffffffu : 0u;
+            cur.x |= c4[i].x & m;
+            cur.y |= c4[i].y & m;
+            cur.z |= c4[i].z & m;
+            cur.w |= c4[i].w & m;
+            if (here) { r_hit = g_hit * 4 + i; cum_v = cum; rank_v = rank; }
+            cum += vt;
+            rank += tv;
+        }
+        uint64_t c2 = cum_v;
+        uint32_t rk = rank_v;
 #pragma unroll 1
         for (int j = 0; j < 8; ++j) {
-            const uint64_t wj = entry_mass(j, rank);
-            cum += wj;
-            if (cum > tau) { ds.hit = base + j; ds.pick_w = wj; break; }
+            const uint32_t word = j < 4 ? (j < 2 ? cur.x : cur.y) : (j < 6 ? cur.z : cur.w);
+            const uint32_t k = (word >> ((j & 1) * 16)) & 0xffffu;
+            const uint64_t wj = (ties && k == tie_key) ? ((rk++ < r_cut) ? w_tie : 0ull) : mass(k);
+            c2 += wj;
+            if (c2 > tau) { ds.hit = (tid * vpl + r_hit) * 8 + j; ds.pick_w = wj; break; }
         }
+    }
+    if (any_tail && has_tail && tail_before <= tau && tau < tail_before + tail_mass) {
+        ds.hit = tail_index;
+        ds.pick_w = tail_mass;
     }
     __syncthreads();
     if (tid == 0) {
@@ -757,20 +758,17 @@ __device__ __forceinline__ void resident_draw(DenseScalars &ds, const uint4 (&he
 
 // Reads the row into registers as 16-bit keys of the scaled entries; returns the lane's largest key.
 template <typename T, bool HAS_T>
-__device__ __forceinline__ uint32_t resident_load_keys_t(const typename T::raw_t *rp, int vocab, int nvec, float temp,
-                                                         uint4 (&held)[RES_VECS], uint32_t *tail_key,
+__device__ __forceinline__ uint32_t resident_load_keys_t(const typename T::raw_t *rp, int vocab, int vpl, int nvec,
+                                                         float temp, uint4 (&held)[RES_VECS], uint32_t *tail_key,
                                                          bool *has_tail) {
     const int tid = threadIdx.x;
-    const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+    const uint4 *vp = reinterpret_cast<const uint4 *>(rp) + tid * vpl;
 #pragma unroll
-    for (int r = 0; r < RES_VECS; ++r) {
-        const int v = tid + r * S_THREADS;
-        held[r] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
-    }
+    for (int r = 0; r < RES_VECS; ++r) held[r] = lane_has_vec(r, vpl, nvec) ? vp[r] : make_uint4(0, 0, 0, 0);
     uint32_t kmax = 0;
 #pragma unroll
     for (int r = 0; r < RES_VECS; ++r) {
-        if (tid + r * S_THREADS < nvec) {
+        if (lane_has_vec(r, vpl, nvec)) {
             // explicit shifts (no 16-bit pointer accesses): the vectors must stay in registers
             const uint32_t in[4] = {held[r].x, held[r].y, held[r].z, held[r].w};
             uint32_t o[4];
@@ -792,11 +790,11 @@ __device__ __forceinline__ uint32_t resident_load_keys_t(const typename T::raw_t
     return kmax;
 }
 template <typename T>
-__device__ __forceinline__ uint32_t resident_load_keys(const typename T::raw_t *rp, int vocab, int nvec, float temp,
-                                                       bool has_t, uint4 (&held)[RES_VECS], uint32_t *tail_key,
-                                                       bool *has_tail) {
-    return has_t ? resident_load_keys_t<T, true>(rp, vocab, nvec, temp, held, tail_key, has_tail)
-                 : resident_load_keys_t<T, false>(rp, vocab, nvec, temp, held, tail_key, has_tail);
+__device__ __forceinline__ uint32_t resident_load_keys(const typename T::raw_t *rp, int vocab, int vpl, int nvec,
+                                                       float temp, bool has_t, uint4 (&held)[RES_VECS],
+                                                       uint32_t *tail_key, bool *has_tail) {
+    return has_t ? resident_load_keys_t<T, true>(rp, vocab, vpl, nvec, temp, held, tail_key, has_tail)
+                 : resident_load_keys_t<T, false>(rp, vocab, vpl, nvec, temp, held, tail_key, has_tail);
 }
 
 template <typename T>
@@ -813,10 +811,12 @@ __device__ __forceinline__ bool nofilter_resident(DenseScalars &ds, const typena
     uint4 held[RES_VECS];
     uint32_t tail_key;
     bool has_tail;
-    const uint32_t lmax = resident_load_keys<T>(rp, vocab, nvec, temp, has_t, held, &tail_key, &has_tail);
+    const int vpl = (nvec + S_THREADS - 1) / S_THREADS;
+    const uint32_t lmax = resident_load_keys<T>(rp, vocab, vpl, nvec, temp, has_t, held, &tail_key, &has_tail);
     const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);
     const float vmax = value_of_key16<T>(kmax);
-    resident_draw<true>(ds, held, tail_key, has_tail, nvec, nvec * 8 + int(threadIdx.x), u, false, 0u, 0xffffffffu, 0ull,
+    resident_draw<true>(ds, held, vpl, nvec, tail_key, has_tail, nvec * 8 + int(threadIdx.x), vocab != nvec * 8, u, false,
+                        0u, 0xffffffffu, 0ull,
                   [&](uint32_t k) { return weight_fix(k == kmax ? 0.0f : value_of_key16<T>(k) - vmax); }, out_slot,
                   lp_slot);
     return true;
@@ -829,40 +829,92 @@ __device__ __forceinline__ int hist_slot(int word) {
     return word ^ ((word >> 4) & 0x1c);  // chunk index (bits 2..4) ^= bits 1..3 of the block index (bits 6..8)
 }
 
-template <typename T>
-__device__ __forceinline__ bool dense_resident(unsigned char *lds, const typename T::raw_t *rp, int vocab, bool vec,
-                                               float temp, bool has_t, bool use_k, int top_k, bool use_p, float top_p,
-                                               float u, int64_t *out_slot, float *lp_slot) {
+// Walks the vectors of this wavefront's share of the row: wavefront w owns the vectors [w * vpw, (w + 1) * vpw)
+// (a contiguous sixteenth of the row, so index order is (wavefront, step, lane, entry)), lane l takes the
+// vectors l, l + 64, ... of that share: every load instruction covers 1 KB of consecutive memory.  Calls
+// f(valid, keys) once per step with the eight 16-bit keys of the lane's vector; the trip count is the same for
+// all lanes, so f may contain wavefront-wide exchanges.  Four loads are in flight per lane.
+template <typename T, bool HAS_T, typename F>
+__device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, float temp, F &&f) {
+    const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll 1
+    for (int i0 = 0; i0 < n_here; i0 += 4 * kWave) {
+        uint4 q[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int idx = i0 + s * kWave + lane;
+            q[s] = idx < n_here ? vp[idx] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            if (i0 + s * kWave < n_here) {  // wavefront-uniform
+                const uint32_t in[4] = {q[s].x, q[s].y, q[s].z, q[s].w};
+                uint32_t k[8];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    k[2 * c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp);
+                    k[2 * c + 1] = elem_key16<T, HAS_T>(in[c] >> 16, temp);
+                }
+                f(i0 + s * kWave + lane < n_here, k);
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+// Exclusive prefix sums over the 64 lanes of a wavefront.
+template <typename V> __device__ __forceinline__ V wave_excl_scan(V v) {
+    const int lane = threadIdx.x & (kWave - 1);
+    V inc = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const V t = __shfl_up(inc, off, kWave);
+        if (lane >= off) inc += t;
+    }
+    return inc - v;
+}
+
+template <typename T, bool HAS_T>
+__device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename T::raw_t *rp, int vocab, bool vec,
+                                             float temp, bool use_k, int top_k, bool use_p, float top_p, float u,
+                                             int64_t *out_slot, float *lp_slot) {
     if (!resident_ok<T>(vocab, vec)) return false;
     uint32_t *hist = reinterpret_cast<uint32_t *>(lds);
     uint32_t *list = hist + D_WORDS;                                   // (key << 16) | count, descending keys
     uint64_t *table = reinterpret_cast<uint64_t *>(list);              // later: mass of key kcut16 + i
     DenseScalars &ds = *reinterpret_cast<DenseScalars *>(list + D_LIST_CAP);
     const int tid = threadIdx.x;
+    const int wave = tid / kWave;
     const int nvec = vocab / 8;
+    const int vpw = (nvec + S_WAVES - 1) / S_WAVES;                    // vectors per wavefront
+    const int v0 = wave * vpw;
+    const int n_here = nvec - v0 < vpw ? (nvec - v0 > 0 ? nvec - v0 : 0) : vpw;
+    const uint4 *vp = reinterpret_cast<const uint4 *>(rp) + v0;
+    // the ragged tail of the row: fewer than 8 entries after the last vector, one per lane of wavefront 0
+    const int tail_index = nvec * 8 + tid;
+    const bool has_tail = tail_index < vocab;
+    const uint32_t tail_key = has_tail ? elem_key16<T, HAS_T>(uint32_t(rp[tail_index]), temp) : 0u;
 
-    // ---- 1. keys into registers, counts into the histogram ------------------------------------------------
+    // ---- 1. counts of the scaled keys into the histogram ----------------------------------------------------
     {
         uint4 *h4 = reinterpret_cast<uint4 *>(hist);
         for (int i = tid; i < D_WORDS / 4; i += S_THREADS) h4[i] = make_uint4(0, 0, 0, 0);
     }
     __syncthreads();
-    uint4 held[RES_VECS];
-    uint32_t tail_key;
-    bool has_tail;
-    const uint32_t lmax = resident_load_keys<T>(rp, vocab, nvec, temp, has_t, held, &tail_key, &has_tail);
+    uint32_t lmax = tail_key;
+    for_wave_vectors<T, HAS_T>(vp, n_here, temp, [&](bool valid, const uint32_t (&k)[8]) {
+        if (valid) {
 #pragma unroll
-    for (int r = 0; r < RES_VECS; ++r) {
-        if (tid + r * S_THREADS < nvec) {
-            const uint32_t in[4] = {held[r].x, held[r].y, held[r].z, held[r].w};
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t k0 = in[q] & 0xffffu, k1 = in[q] >> 16;
-                atomicAdd(&hist[hist_slot(k0 >> 1)], (k0 & 1) ? 0x10000u : 1u);
-                atomicAdd(&hist[hist_slot(k1 >> 1)], (k1 & 1) ? 0x10000u : 1u);
+            for (int j = 0; j < 8; ++j) {
+                atomicAdd(&hist[hist_slot(k[j] >> 1)], (k[j] & 1) ? 0x10000u : 1u);
+                lmax = k[j] > lmax ? k[j] : lmax;
             }
         }
-    }
+    });
     if (has_tail) atomicAdd(&hist[hist_slot(tail_key >> 1)], (tail_key & 1) ? 0x10000u : 1u);
     const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);  // its barriers also publish the histogram
     const float vmax = value_of_key16<T>(kmax);
@@ -1016,10 +1068,148 @@ __device__ __forceinline__ bool dense_resident(unsigned char *lds, const typenam
     }
     __syncthreads();
     // ---- 7. draw over the survivors in index order ------------------------------------------------------------
-    (void)z_kept;  // equals the sum of the tile masses below
+    (void)z_kept;  // equals the total computed from the table below
     const uint32_t first = track_ties ? kcut16 + 1 : kcut16;  // lowest key whose entries all survive
-    resident_draw<false>(ds, held, tail_key, has_tail, nvec, nvec * 8 + tid, u, track_ties, kcut16, r_cut, w_tie,
-                  [&](uint32_t k) { return table[k >= first ? k - kcut16 : span]; }, out_slot, lp_slot);
+    auto mass = [&](uint32_t k) { return table[k >= first ? k - kcut16 : span]; };
+    auto is_tie = [&](uint32_t k) { return track_ties && k == kcut16; };
+    // 7a. per wavefront: mass of the full survivors and number of tie-group entries of its share of the row
+    {
+        uint64_t m = 0;
+        uint32_t t = 0;
+        for_wave_vectors<T, HAS_T>(vp, n_here, temp, [&](bool valid, const uint32_t (&k)[8]) {
+            if (valid) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    m += mass(k[j]);
+                    t += is_tie(k[j]) ? 1u : 0u;
+                }
+            }
+        });
+        m = wave_sum_u64(m);
+        t = wave_sum_u32(t);
+        uint64_t mt = has_tail ? mass(tail_key) : 0ull;
+        uint32_t tt = (has_tail && is_tie(tail_key)) ? 1u : 0u;
+        if (wave == 0) {
+            mt = wave_sum_u64(mt);
+            tt = wave_sum_u32(tt);
+        }
+        if ((tid & (kWave - 1)) == 0) {
+            ds.seg_mass[wave] = m;
+            ds.seg_ties[wave] = t;
+            if (wave == 0) {
+                ds.seg_mass[S_WAVES] = mt;
+                ds.seg_ties[S_WAVES] = tt;
+                ds.hit = -1;
+            }
+        }
+    }
+    __syncthreads();
+    // 7b. the segment (a wavefront's share, or the tail) that holds floor(u * Z)
+    uint64_t z = 0;
+    {
+        uint32_t seen = 0;
+#pragma unroll
+        for (int g = 0; g <= S_WAVES; ++g) {
+            const uint32_t t = ds.seg_ties[g];
+            const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
+            z += ds.seg_mass[g] + uint64_t(t < room ? t : room) * w_tie;
+            seen += t;
+        }
+    }
+    const uint64_t tau = floor_scale(u, z);
+    uint64_t acc = 0;          // mass before the segment
+    uint32_t ties_before = 0;  // tie-group entries before the segment
+    int seg = -1;
+    {
+        uint32_t seen = 0;
+#pragma unroll
+        for (int g = 0; g <= S_WAVES; ++g) {
+            const uint32_t t = ds.seg_ties[g];
+            const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
+            const uint64_t m = ds.seg_mass[g] + uint64_t(t < room ? t : room) * w_tie;
+            if (seg < 0 && tau < acc + m) { seg = g; ties_before = seen; }
+            if (seg < 0) acc += m;
+            seen += t;
+        }
+    }
+    // 7c. inside the segment: the step, the lane, the entry (one wavefront works, the others wait at the barrier)
+    if (seg == wave) {
+        uint64_t cum = acc;
+        uint32_t rank = ties_before;
+        bool found = false;
+        uint32_t hk[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // this lane's keys in the step that holds tau
+        bool hvalid = false;
+        int hstep = 0, step = 0;
+        uint64_t hcum = 0;
+        uint32_t hrank = 0;
+        for_wave_vectors<T, HAS_T>(vp, n_here, temp, [&](bool valid, const uint32_t (&k)[8]) {
+            uint64_t m = 0;
+            uint32_t t = 0;
+            if (valid) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    m += mass(k[j]);
+                    t += is_tie(k[j]) ? 1u : 0u;
+                }
+            }
+            const uint64_t ms = wave_sum_u64(m);
+            const uint32_t ts = wave_sum_u32(t);
+            const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
+            const uint64_t total = ms + uint64_t(ts < room ? ts : room) * w_tie;
+            if (!found && tau < cum + total) {  // wavefront-uniform
+                found = true;
+                hstep = step;
+                hcum = cum;
+                hrank = rank;
+                hvalid = valid;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) hk[j] = k[j];
+            }
+            cum += total;
+            rank += ts;
+            ++step;
+        });
+        // lanes of that step in order: tie ranks first, then masses
+        uint32_t lt = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) lt += (hvalid && is_tie(hk[j])) ? 1u : 0u;
+        uint32_t rk = hrank + wave_excl_scan<uint32_t>(lt);
+        const uint32_t rk0 = rk;
+        uint64_t lm = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (hvalid) lm += is_tie(hk[j]) ? ((rk++ < r_cut) ? w_tie : 0ull) : mass(hk[j]);
+        const uint64_t before = hcum + wave_excl_scan<uint64_t>(lm);
+        if (before <= tau && tau < before + lm) {
+            uint64_t c2 = before;
+            uint32_t r2 = rk0;
+            bool done = false;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint64_t wj = is_tie(hk[j]) ? ((r2++ < r_cut) ? w_tie : 0ull) : mass(hk[j]);
+                c2 += wj;
+                if (!done && c2 > tau) {
+                    done = true;
+                    ds.hit = (v0 + hstep * kWave + (tid & (kWave - 1))) * 8 + j;
+                    ds.pick_w = wj;
+                }
+            }
+        }
+    } else if (seg == S_WAVES && wave == 0) {
+        const bool tie = has_tail && is_tie(tail_key);
+        const uint32_t rk = ties_before + wave_excl_scan<uint32_t>(tie ? 1u : 0u);
+        const uint64_t wt = has_tail ? (tie ? (rk < r_cut ? w_tie : 0ull) : mass(tail_key)) : 0ull;
+        const uint64_t before = acc + wave_excl_scan<uint64_t>(wt);
+        if (before <= tau && tau < before + wt) {
+            ds.hit = tail_index;
+            ds.pick_w = wt;
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        *out_slot = ds.hit;
+        if (lp_slot != nullptr) *lp_slot = ds.hit >= 0 ? log_ratio(ds.pick_w, z) : __builtin_nanf("");
+    }
     return true;
 }
 
@@ -1091,8 +1281,11 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
         }
     } else if (!no_fast) {
         if constexpr (DENSE && T::kBytes == 2) {
-            if (dense_resident<T>(lds, rp, vocab, vec, temp, has_t, use_k, top_k, use_p, top_p, u, out + row, lp_slot))
-                return;
+            const bool done = has_t ? dense_stream<T, true>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
+                                                            out + row, lp_slot)
+                                    : dense_stream<T, false>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
+                                                             out + row, lp_slot);
+            if (done) return;
             __syncthreads();
         }
     }
