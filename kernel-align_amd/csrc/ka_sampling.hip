@@ -155,7 +155,7 @@ struct DenseScalars {
     uint64_t seg_mass[S_WAVES + 1];  // dense path: mass of each wavefront's share of the row, and of the ragged tail
     uint32_t seg_ties[S_WAVES + 1];  // ... and its number of tie-group entries
     uint64_t z_topk, before_cut, w_cut, pick_w;
-    uint32_t i_topk, n_cut, kcut16;
+    uint32_t i_topk, n_cut, kcut16, i_last, tie_hi, tie_lo, fail;
     int best_i;
     int64_t hit;
 };
@@ -897,16 +897,17 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     // the ragged tail of the row: fewer than 8 entries after the last vector, one per lane of wavefront 0
     const int tail_index = nvec * 8 + tid;
     const bool has_tail = tail_index < vocab;
-    const uint32_t tail_key = has_tail ? elem_key16<T, HAS_T>(uint32_t(rp[tail_index]), temp) : 0u;
+    const uint32_t tail_key = has_tail ? elem_key16<T, false>(uint32_t(rp[tail_index]), 1.0f) : 0u;
 
-    // ---- 1. counts of the scaled keys into the histogram ----------------------------------------------------
+    // ---- 1. counts of the raw keys (no temperature yet: the scaling x -> round(x / T) is monotone, so it can be
+    //         applied to the few thousand occupied keys instead of to every entry) into the histogram ----------
     {
         uint4 *h4 = reinterpret_cast<uint4 *>(hist);
         for (int i = tid; i < D_WORDS / 4; i += S_THREADS) h4[i] = make_uint4(0, 0, 0, 0);
     }
     __syncthreads();
     uint32_t lmax = tail_key;
-    for_wave_vectors<T, HAS_T>(vp, n_here, temp, [&](bool valid, const uint32_t (&k)[8]) {
+    for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
         if (valid) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -916,8 +917,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         }
     });
     if (has_tail) atomicAdd(&hist[hist_slot(tail_key >> 1)], (tail_key & 1) ? 0x10000u : 1u);
-    const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);  // its barriers also publish the histogram
-    const float vmax = value_of_key16<T>(kmax);
+    const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);  // largest raw key; the barriers also publish the histogram
 
     // ---- 2. compact the occupied keys, in descending order, into the list ---------------------------------
     // lane t owns the words [D_WORDS - 32 (t + 1), D_WORDS - 32 t) and walks them from the top
@@ -956,8 +956,17 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     }
     __syncthreads();
 
-    // ---- 3. masses, once per occupied key: lane t takes the entries [t * D_PER_THREAD, ...) ---------------
-    uint32_t ent[D_PER_THREAD];
+    // ---- 3. scaled key and mass, once per occupied key: lane t takes the entries [t * D_PER_THREAD, ...) -------
+    // Several raw keys may scale to one value; such a run of entries is one tie group of the operator.
+    uint16_t *const skl = reinterpret_cast<uint16_t *>(hist);  // scaled key of every list entry (the counts are spent)
+    auto scaled = [&](uint32_t raw_key) -> uint32_t {
+        if (!HAS_T) return raw_key;
+        const uint32_t bits = (raw_key & 0x8000u) ? (raw_key & 0x7fffu) : (~raw_key & 0xffffu);
+        return elem_key16<T, true>(bits, temp);
+    };
+    const uint32_t kmax_s = scaled(kmax);
+    const float vmax = value_of_key16<T>(kmax_s);
+    uint32_t ent[D_PER_THREAD], sk[D_PER_THREAD];
     uint64_t wgt[D_PER_THREAD];
     uint64_t m_local = 0;
     uint32_t c_local = 0;
@@ -965,48 +974,67 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     for (int e = 0; e < D_PER_THREAD; ++e) {
         const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
         ent[e] = i < occ_total ? list[i] : 0u;
-        const uint32_t k = ent[e] >> 16, c = ent[e] & 0xffffu;
-        wgt[e] = c ? weight_fix(k == kmax ? 0.0f : value_of_key16<T>(k) - vmax) : 0ull;
+        const uint32_t c = ent[e] & 0xffffu;
+        sk[e] = scaled(ent[e] >> 16);
+        wgt[e] = c ? weight_fix(sk[e] == kmax_s ? 0.0f : value_of_key16<T>(sk[e]) - vmax) : 0ull;
         m_local += wgt[e] * c;
         c_local += c;
+        if (i < occ_total) skl[i] = uint16_t(sk[e]);
     }
     uint64_t z_all;
     uint32_t c_all;
     const uint64_t m_before = block_excl_scan<uint64_t>(m_local, ds.wave_u64, &z_all);
     const uint32_t c_before = block_excl_scan<uint32_t>(c_local, ds.wave_u32, &c_all);
-
-    // ---- 4. top-k: the list entry that holds the top_k-th largest entry; everything down to it survives ----
     if (tid == 0) {
         ds.i_topk = occ_total - 1;
         ds.z_topk = z_all;
         ds.best_i = -1;
+        ds.fail = 0;
     }
-    __syncthreads();
-    if (use_k && c_before < uint32_t(top_k) && uint32_t(top_k) <= c_before + c_local) {
-        uint32_t c_run = c_before;
-        uint64_t m_run = m_before;
+    __syncthreads();  // skl[] complete
+    // last entry of the run (equal scaled keys) that contains entry i; a run longer than 64 entries (a huge
+    // temperature folds many values together) is left to the radix path
+    auto run_end = [&](uint32_t i) -> uint32_t {
+        const uint32_t key = skl[i];
+        uint32_t j = i;
+        int guard = 0;
+        while (j + 1 < occ_total && skl[j + 1] == key && guard < 64) { ++j; ++guard; }
+        if (guard == 64) ds.fail = 1;
+        return j;
+    };
+
+    // ---- 4. top-k: the run that holds the top_k-th largest entry; everything down to its end survives ----------
+    if (use_k) {
+        if (c_before < uint32_t(top_k) && uint32_t(top_k) <= c_before + c_local) {
+            uint32_t c_run = c_before;
 #pragma unroll
-        for (int e = 0; e < D_PER_THREAD; ++e) {
-            const uint32_t c = ent[e] & 0xffffu;
-            const bool here = c_run < uint32_t(top_k) && uint32_t(top_k) <= c_run + c;
-            c_run += c;
-            m_run += wgt[e] * c;
-            if (here) {
-                ds.i_topk = uint32_t(tid) * D_PER_THREAD + e;
-                ds.z_topk = m_run;
+            for (int e = 0; e < D_PER_THREAD; ++e) {
+                const uint32_t c = ent[e] & 0xffffu;
+                if (c_run < uint32_t(top_k) && uint32_t(top_k) <= c_run + c) ds.i_topk = run_end(uint32_t(tid) * D_PER_THREAD + e);
+                c_run += c;
             }
         }
+        __syncthreads();
+        if (ds.i_topk / D_PER_THREAD == uint32_t(tid)) {  // mass of everything down to that entry
+            uint64_t m_run = m_before;
+#pragma unroll
+            for (int e = 0; e < D_PER_THREAD; ++e) {
+                m_run += wgt[e] * (ent[e] & 0xffffu);
+                if (uint32_t(tid) * D_PER_THREAD + e == ds.i_topk) ds.z_topk = m_run;
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     const uint32_t i_topk = ds.i_topk;
     const uint64_t z_topk = ds.z_topk;
 
-    // ---- 5. top-p: the last entry at or above i_topk whose first element has (mass before it) <= theta -----
-    uint32_t i_cut = i_topk;
+    // ---- 5. top-p: the last run at or above i_topk whose first element has (mass before it) <= theta ----------
+    uint32_t i_last = i_topk;       // last surviving list entry
     uint64_t z_kept = z_topk;
     bool track_ties = false;
     uint32_t r_cut = 0xffffffffu;
     uint64_t w_tie = 0;
+    uint32_t tie_hi = 0, tie_lo = 0;  // raw keys of the tie group that is cut
     if (use_p) {
         const uint64_t theta = floor_scale(top_p, z_topk);
         int best = -1;
@@ -1015,21 +1043,29 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         for (int e = 0; e < D_PER_THREAD; ++e) {
             const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
             const uint32_t c = ent[e] & 0xffffu;
-            if (c != 0 && i <= i_topk && m_run <= theta) best = int(i);
+            const uint32_t prev = e > 0 ? sk[e - 1] : (i > 0 && i < occ_total ? uint32_t(skl[i - 1]) : 0xffffffffu);
+            const bool start = i == 0 || prev != sk[e];
+            if (c != 0 && start && i <= i_topk && m_run <= theta) best = int(i);
             m_run += wgt[e] * c;
         }
         if (best >= 0) atomicMax(&ds.best_i, best);
         __syncthreads();
-        i_cut = uint32_t(ds.best_i);
+        const uint32_t i_cut = uint32_t(ds.best_i);
         if (i_cut / D_PER_THREAD == uint32_t(tid)) {
             uint64_t m_run2 = m_before;
 #pragma unroll
             for (int e = 0; e < D_PER_THREAD; ++e) {
                 const uint32_t c = ent[e] & 0xffffu;
                 if (uint32_t(tid) * D_PER_THREAD + e == i_cut) {
+                    const uint32_t j_end = run_end(i_cut);
+                    uint32_t n = 0;
+                    for (uint32_t j = i_cut; j <= j_end; ++j) n += list[j] & 0xffffu;
                     ds.before_cut = m_run2;
                     ds.w_cut = wgt[e];
-                    ds.n_cut = c;
+                    ds.n_cut = n;
+                    ds.i_last = j_end;
+                    ds.tie_hi = ent[e] >> 16;
+                    ds.tie_lo = list[j_end] >> 16;
                 }
                 m_run2 += wgt[e] * c;
             }
@@ -1037,6 +1073,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         __syncthreads();
         const uint64_t before = ds.before_cut, w_cut = ds.w_cut;
         const uint64_t n_cut = ds.n_cut;
+        i_last = ds.i_last;
         uint64_t r = n_cut;
         if (w_cut > 0) {
             const uint64_t fit = (theta - before) / w_cut + 1;  // entries t with before + t * w <= theta
@@ -1047,13 +1084,16 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
             track_ties = true;
             r_cut = uint32_t(r);
             w_tie = w_cut;
+            tie_hi = ds.tie_hi;
+            tie_lo = ds.tie_lo;
         }
     }
-    // ---- 6. masses of the surviving keys into a table indexed by key - cut key ------------------------------
-    if (tid == i_cut / D_PER_THREAD) {
+    if (ds.fail) return false;
+    // ---- 6. masses of the surviving raw keys into a table indexed by key - lowest surviving key ---------------
+    if (tid == i_last / D_PER_THREAD) {
 #pragma unroll
         for (int e = 0; e < D_PER_THREAD; ++e)
-            if (uint32_t(tid) * D_PER_THREAD + e == i_cut) ds.kcut16 = ent[e] >> 16;
+            if (uint32_t(tid) * D_PER_THREAD + e == i_last) ds.kcut16 = ent[e] >> 16;
     }
     __syncthreads();  // also: every lane is done reading the list
     const uint32_t kcut16 = ds.kcut16;
@@ -1064,19 +1104,19 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
 #pragma unroll
     for (int e = 0; e < D_PER_THREAD; ++e) {
         const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
-        if (i <= i_cut && (ent[e] & 0xffffu) != 0) table[(ent[e] >> 16) - kcut16] = wgt[e];
+        if (i <= i_last && (ent[e] & 0xffffu) != 0) table[(ent[e] >> 16) - kcut16] = wgt[e];
     }
     __syncthreads();
     // ---- 7. draw over the survivors in index order ------------------------------------------------------------
     (void)z_kept;  // equals the total computed from the table below
-    const uint32_t first = track_ties ? kcut16 + 1 : kcut16;  // lowest key whose entries all survive
+    const uint32_t first = track_ties ? tie_hi + 1 : kcut16;  // lowest raw key whose entries all survive
     auto mass = [&](uint32_t k) { return table[k >= first ? k - kcut16 : span]; };
-    auto is_tie = [&](uint32_t k) { return track_ties && k == kcut16; };
+    auto is_tie = [&](uint32_t k) { return track_ties && k >= tie_lo && k <= tie_hi; };
     // 7a. per wavefront: mass of the full survivors and number of tie-group entries of its share of the row
     {
         uint64_t m = 0;
         uint32_t t = 0;
-        for_wave_vectors<T, HAS_T>(vp, n_here, temp, [&](bool valid, const uint32_t (&k)[8]) {
+        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
             if (valid) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -1142,7 +1182,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         int hstep = 0, step = 0;
         uint64_t hcum = 0;
         uint32_t hrank = 0;
-        for_wave_vectors<T, HAS_T>(vp, n_here, temp, [&](bool valid, const uint32_t (&k)[8]) {
+        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
             uint64_t m = 0;
             uint32_t t = 0;
             if (valid) {

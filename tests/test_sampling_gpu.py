@@ -292,3 +292,15 @@ def test_randomised_shapes_modes_and_value_grids(sampler, seed):
         want = exact.sample(logits, temp, k, p, u)
         assert torch.equal(got, want), (f"trial {trial}: vocab={vocab} dtype={dtype} grid={grid} spread={spread:.2f} "
                                         f"k={k} p={p} T={temp}: rows {(got != want).nonzero().flatten().tolist()}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_temperature_merges_raw_values_into_tie_groups(sampler, dtype):
+    """The histogram path counts raw values and scales only the occupied ones; raw values that round to the
+    same scaled value must act as one tie group (top-k ties kept, top-p cut by index order across them)."""
+    g = torch.Generator().manual_seed(51)
+    u = torch.rand(12, generator=g)
+    for spread, temp in [(3.0, 3.0), (3.0, 25.0), (0.5, 7.0), (6.0, 1000.0), (3.0, 0.31)]:
+        logits = (torch.randn(12, 30000, generator=g) * spread).to(dtype)
+        for k, p in [(None, 0.9), (None, 0.3), (2000, None), (1500, 0.95), (None, 0.999)]:
+            check_exact(sampler, logits, u, k, p, temp)
