@@ -341,9 +341,38 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     constexpr int RES_VECS = 16;
     const int nvec = vocab / EPV;
     const bool resident = vec && T::kDtype == KA_DTYPE_BF16 && nvec <= RES_VECS * S_THREADS;
+    // A longer or wider row (fp32: up to 131,072 entries) does not fit in registers, but the maximum of each of
+    // the lane's vectors does: the collection pass then re-reads only the few vectors that hold a candidate.
+    constexpr int TRK_VECS = 32;
+    const bool tracked = vec && !resident && nvec <= TRK_VECS * S_THREADS;
     uint4 held[RES_VECS];
+    float vmaxs[TRK_VECS];
     float lmaxf = -__builtin_inff();
-    if (resident) {
+    if (tracked) {
+        const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+#pragma unroll
+        for (int g = 0; g < TRK_VECS / 8; ++g) {
+            uint4 q[8];
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const int v = tid + (g * 8 + s) * S_THREADS;
+                q[s] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                float vm = -__builtin_inff();
+                if (tid + (g * 8 + s) * S_THREADS < nvec) {
+                    const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[s]);
+#pragma unroll
+                    for (int j = 0; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
+                }
+                vmaxs[g * 8 + s] = vm;
+                lmaxf = fmaxf(lmaxf, vm);
+            }
+        }
+        const int i = nvec * EPV + tid;  // ragged tail of the row
+        if (i < vocab) lmaxf = fmaxf(lmaxf, T::widen(rp[i]));
+    } else if (resident) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll
         for (int r = 0; r < RES_VECS; ++r) {
@@ -424,6 +453,20 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
 #pragma unroll
                     for (int j = 0; j < EPV; ++j) collect(v * EPV + j, e[j]);
                 }
+            }
+        }
+        const int i = nvec * EPV + tid;
+        if (i < vocab) collect(i, rp[i]);
+    } else if (tracked) {
+        const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+#pragma unroll
+        for (int r = 0; r < TRK_VECS; ++r) {
+            if (vmaxs[r] >= boundf) {  // rare: about top_k vectors of the whole row hold a candidate
+                const int v = tid + r * S_THREADS;
+                const uint4 q = vp[v];
+                const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) collect(v * EPV + j, e[j]);
             }
         }
         const int i = nvec * EPV + tid;
