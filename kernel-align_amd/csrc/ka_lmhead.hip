@@ -53,9 +53,6 @@ struct Partial {
 // swz(row) = (row >> 1) & 7; measured with a ds_read_b128 micro-benchmark on gfx950 this pattern reads at
 // the same rate as a contiguous one, while (row & 7) and an unswizzled slab cost 1.5x and 4.5x.
 __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
-__device__ __forceinline__ int slab_offset(int row, int chunk) {
-    return row * LM_BK + ((chunk ^ swz(row)) << 3);  // in bf16 elements
-}
 
 typedef __attribute__((address_space(3))) void lds_void;
 
