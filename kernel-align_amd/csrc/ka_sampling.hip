@@ -923,7 +923,7 @@ template <typename V> __device__ __forceinline__ V wave_excl_scan(V v) {
     return inc - v;
 }
 
-template <typename T, bool HAS_T>
+template <typename T, bool HAS_T, bool ALL_SURVIVE>
 __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename T::raw_t *rp, int vocab, bool vec,
                                              float temp, bool use_k, int top_k, bool use_p, float top_p, float u,
                                              int64_t *out_slot, float *lp_slot) {
@@ -934,6 +934,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     DenseScalars &ds = *reinterpret_cast<DenseScalars *>(list + D_LIST_CAP);
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
+    constexpr bool all_survive = ALL_SURVIVE;  // no filter at all (the caller passes use_k = use_p = false)
     const int nvec = vocab / 8;
     const int vpw = (nvec + S_WAVES - 1) / S_WAVES;                    // vectors per wavefront
     const int v0 = wave * vpw;
@@ -1024,7 +1025,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         wgt[e] = c ? weight_fix(sk[e] == kmax_s ? 0.0f : value_of_key16<T>(sk[e]) - vmax) : 0ull;
         m_local += wgt[e] * c;
         c_local += c;
-        if (i < occ_total) skl[i] = uint16_t(sk[e]);
+        if (i < occ_total && !all_survive) skl[i] = uint16_t(sk[e]);
     }
     uint64_t z_all;
     uint32_t c_all;
@@ -1048,6 +1049,29 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         return j;
     };
 
+    // ---- the draw over the survivors in index order; mass(key) is the integer mass of an entry that survives
+    //      entirely (0 otherwise), is_tie(key) marks the entries of a tie group of which only the first r_cut
+    //      (in index order) survive, each with mass w_tie -------------------------------------------------------
+    bool track_ties = false;
+    uint32_t r_cut = 0xffffffffu;
+    uint64_t w_tie = 0;
+    uint32_t tie_hi = 0, tie_lo = 0;  // raw keys of the tie group that is cut
+
+    // ---- no filter: every occupied key survives; its mass is found through the key's list index ---------------
+    uint16_t *const idx16 = reinterpret_cast<uint16_t *>(hist);  // list index of every occupied raw key
+    uint32_t kcut16 = 0, span = 0, first = 0;
+    if (all_survive) {
+        if (occ_total > uint32_t(D_TABLE_CAP)) return false;  // the mass table holds 8 bytes per occupied key
+#pragma unroll
+        for (int e = 0; e < D_PER_THREAD; ++e) {
+            const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;
+            if (i < occ_total) {
+                idx16[ent[e] >> 16] = uint16_t(i);
+                table[i] = wgt[e];  // every lane has read its list entries (barrier above)
+            }
+        }
+        __syncthreads();
+    } else {
     // ---- 4. top-k: the run that holds the top_k-th largest entry; everything down to its end survives ----------
     if (use_k) {
         if (c_before < uint32_t(top_k) && uint32_t(top_k) <= c_before + c_local) {
@@ -1076,10 +1100,6 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     // ---- 5. top-p: the last run at or above i_topk whose first element has (mass before it) <= theta ----------
     uint32_t i_last = i_topk;       // last surviving list entry
     uint64_t z_kept = z_topk;
-    bool track_ties = false;
-    uint32_t r_cut = 0xffffffffu;
-    uint64_t w_tie = 0;
-    uint32_t tie_hi = 0, tie_lo = 0;  // raw keys of the tie group that is cut
     if (use_p) {
         const uint64_t theta = floor_scale(top_p, z_topk);
         int best = -1;
@@ -1141,8 +1161,8 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
             if (uint32_t(tid) * D_PER_THREAD + e == i_last) ds.kcut16 = ent[e] >> 16;
     }
     __syncthreads();  // also: every lane is done reading the list
-    const uint32_t kcut16 = ds.kcut16;
-    const uint32_t span = kmax - kcut16 + 1;
+    kcut16 = ds.kcut16;
+    span = kmax - kcut16 + 1;
     if (span >= uint32_t(D_TABLE_CAP)) return false;
     for (uint32_t i = tid; i <= span; i += S_THREADS) table[i] = 0;  // table[span] stays 0: the slot of every non-survivor
     __syncthreads();
@@ -1152,10 +1172,13 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         if (i <= i_last && (ent[e] & 0xffffu) != 0) table[(ent[e] >> 16) - kcut16] = wgt[e];
     }
     __syncthreads();
+    (void)z_kept;  // equals the total the draw computes from the table
+    first = track_ties ? tie_hi + 1 : kcut16;  // lowest raw key whose entries all survive
+    }  // filters
     // ---- 7. draw over the survivors in index order ------------------------------------------------------------
-    (void)z_kept;  // equals the total computed from the table below
-    const uint32_t first = track_ties ? tie_hi + 1 : kcut16;  // lowest raw key whose entries all survive
-    auto mass = [&](uint32_t k) { return table[k >= first ? k - kcut16 : span]; };
+    auto mass = [&](uint32_t k) -> uint64_t {
+        return all_survive ? table[idx16[k]] : table[k >= first ? k - kcut16 : span];
+    };
     auto is_tie = [&](uint32_t k) { return track_ties && k >= tie_lo && k <= tie_hi; };
     // 7a. per wavefront: mass of the full survivors and number of tie-group entries of its share of the row
     {
@@ -1359,19 +1382,25 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (use_k && top_k <= S_THREADS && !no_fast) {
         if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot)) return;
         __syncthreads();
-    } else if (!use_k && !use_p && !no_fast) {
-        if constexpr (T::kBytes == 2) {
-            if (nofilter_resident<T>(sh.ds, rp, vocab, vec, temp, has_t, u, out + row, lp_slot)) return;
-            __syncthreads();
-        }
     } else if (!no_fast) {
         if constexpr (DENSE && T::kBytes == 2) {
-            const bool done = has_t ? dense_stream<T, true>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
+            bool done;
+            if (!use_k && !use_p)
+                done = has_t ? dense_stream<T, true, true>(lds, rp, vocab, vec, temp, false, 0, false, 1.0f, u, out + row, lp_slot)
+                             : dense_stream<T, false, true>(lds, rp, vocab, vec, temp, false, 0, false, 1.0f, u, out + row, lp_slot);
+            else
+                done = has_t ? dense_stream<T, true, false>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
                                                             out + row, lp_slot)
-                                    : dense_stream<T, false>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
+                             : dense_stream<T, false, false>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
                                                              out + row, lp_slot);
             if (done) return;
             __syncthreads();
+        }
+        if constexpr (!DENSE && T::kBytes == 2) {
+            if (!use_k && !use_p) {  // launched without the histogram's LDS: fp16, whose rows hold too many distinct values
+                if (nofilter_resident<T>(sh.ds, rp, vocab, vec, temp, has_t, u, out + row, lp_slot)) return;
+                __syncthreads();
+            }
         }
     }
 
@@ -1596,7 +1625,11 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
     if (T::kBytes == 2 && aligned && !no_fast && vocab / 8 <= RES_VECS * S_THREADS) {
         const bool per_row = prm.top_k_rows != nullptr || prm.top_p_rows != nullptr;
         const bool k_on = prm.top_k > 0 && prm.top_k < vocab;
-        dense = per_row || (k_on && prm.top_k > S_THREADS) || (!k_on && prm.top_p < 1.0f);
+        // (no filter at all: the histogram path for bf16; an fp16 row has too many distinct values for its list and
+        //  takes the register-resident no-filter path of the small-LDS kernel)
+        const bool no_filter = !k_on && !(prm.top_p < 1.0f);
+        dense = per_row || (k_on && prm.top_k > S_THREADS) || (!k_on && !no_filter) ||
+                (no_filter && T::kDtype == KA_DTYPE_BF16);
     }
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const typename T::raw_t *lp = static_cast<const typename T::raw_t *>(logits);
