@@ -157,7 +157,7 @@ struct DenseScalars {
     uint64_t seg_mass[S_WAVES + 1];  // dense path: mass of each wavefront's share of the row, and of the ragged tail
     uint32_t seg_ties[S_WAVES + 1];  // ... and its number of tie-group entries
     uint64_t z_topk, before_cut, w_cut, pick_w;
-    uint32_t i_topk, n_cut, kcut16, i_last, tie_hi, tie_lo, fail;
+    uint32_t i_topk, n_cut, kcut16, i_last, tie_hi, tie_lo, fail, n_inf;
     int best_i;
     int64_t hit;
 };
@@ -952,18 +952,30 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         for (int i = tid; i < D_WORDS / 4; i += S_THREADS) h4[i] = make_uint4(0, 0, 0, 0);
     }
     __syncthreads();
+    // Entries at -inf (a masked vocabulary; NaNs count as -inf) have mass 0 unless the whole row is -inf: they are
+    // counted apart in 32 bits and take no further part, so that a row with more than 65,535 masked entries does
+    // not overflow a 16-bit counter.
+    constexpr uint32_t kNegInfKey = ~(0x8000u | (T::kDtype == KA_DTYPE_BF16 ? 0x7f80u : 0x7c00u)) & 0xffffu;
+    if (tid == 0) ds.n_inf = 0;
     uint32_t lmax = tail_key;
+    uint32_t my_inf = (has_tail && tail_key == kNegInfKey) ? 1u : 0u;
     for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
         if (valid) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                atomicAdd(&hist[hist_slot(k[j] >> 1)], (k[j] & 1) ? 0x10000u : 1u);
+                if (k[j] == kNegInfKey) ++my_inf;
+                else atomicAdd(&hist[hist_slot(k[j] >> 1)], (k[j] & 1) ? 0x10000u : 1u);
                 lmax = k[j] > lmax ? k[j] : lmax;
             }
         }
     });
-    if (has_tail) atomicAdd(&hist[hist_slot(tail_key >> 1)], (tail_key & 1) ? 0x10000u : 1u);
+    if (has_tail && tail_key != kNegInfKey) atomicAdd(&hist[hist_slot(tail_key >> 1)], (tail_key & 1) ? 0x10000u : 1u);
+    my_inf = wave_sum_u32(my_inf);
+    __syncthreads();  // ds.n_inf is zero
+    if ((tid & (kWave - 1)) == 0 && my_inf != 0) atomicAdd(&ds.n_inf, my_inf);
     const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);  // largest raw key; the barriers also publish the histogram
+    if (kmax == kNegInfKey) return false;  // nothing above -inf: the draw is uniform over the row (radix path)
+    const uint32_t n_inf = ds.n_inf;
 
     // ---- 2. compact the occupied keys, in descending order, into the list ---------------------------------
     // lane t owns the words [D_WORDS - 32 (t + 1), D_WORDS - 32 t) and walks them from the top
@@ -988,7 +1000,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     block_excl_scan<uint32_t>(n_cnt, ds.wave_u32, &cnt_total);
     // a 16-bit counter that overflowed loses 65,535 or 65,536 entries of the total; more occupied keys than
     // the list holds: leave the row to the radix path
-    if (cnt_total != uint32_t(vocab) || occ_total > uint32_t(D_LIST_CAP)) return false;
+    if (cnt_total + n_inf != uint32_t(vocab) || occ_total > uint32_t(D_LIST_CAP)) return false;
 #pragma unroll
     for (int c = 7; c >= 0; --c) {
         const uint4 wv = chunk_of(c);
@@ -1061,7 +1073,11 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     uint16_t *const idx16 = reinterpret_cast<uint16_t *>(hist);  // list index of every occupied raw key
     uint32_t kcut16 = 0, span = 0, first = 0;
     if (all_survive) {
-        if (occ_total > uint32_t(D_TABLE_CAP)) return false;  // the mass table holds 8 bytes per occupied key
+        if (occ_total >= uint32_t(D_TABLE_CAP)) return false;  // the mass table holds 8 bytes per occupied key
+        if (tid == 0) {  // the -inf entries look up a zero behind the last occupied key
+            idx16[kNegInfKey] = uint16_t(occ_total);
+            table[occ_total] = 0;
+        }
 #pragma unroll
         for (int e = 0; e < D_PER_THREAD; ++e) {
             const uint32_t i = uint32_t(tid) * D_PER_THREAD + e;

@@ -304,3 +304,22 @@ def test_temperature_merges_raw_values_into_tie_groups(sampler, dtype):
         logits = (torch.randn(12, 30000, generator=g) * spread).to(dtype)
         for k, p in [(None, 0.9), (None, 0.3), (2000, None), (1500, 0.95), (None, 0.999)]:
             check_exact(sampler, logits, u, k, p, temp)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_masked_vocabulary_rows(sampler, dtype):
+    """Constrained decoding masks most of the vocabulary with -inf: more equal entries than a 16-bit histogram
+    counter holds.  Every mode must still return the oracle's ids (and never a masked id)."""
+    g = torch.Generator().manual_seed(61)
+    vocab = 128256
+    logits = (torch.randn(8, vocab, generator=g) * 3).to(dtype)
+    masked = torch.rand(8, vocab, generator=g) < 0.8                       # ~102,600 entries per row
+    logits[masked] = float("-inf")
+    logits[7] = float("-inf")                                              # a fully masked row: uniform draw
+    logits[6, :] = float("-inf"); logits[6, 77] = 1.5                      # one admissible token
+    u = torch.rand(8, generator=g)
+    for k, p, temp in [(None, None, 1.0), (None, 0.9, 0.7), (2000, None, 1.0), (50, 0.9, 0.7), (None, 0.5, 1.3),
+                       (40000, 0.95, 1.0)]:
+        got = check_exact(sampler, logits, u, k, p, temp)
+        assert not masked[torch.arange(6), got[:6]].any()
+        assert got[6] == 77
