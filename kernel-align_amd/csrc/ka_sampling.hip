@@ -877,8 +877,9 @@ __device__ __forceinline__ int hist_slot(int word) {
 // Walks the vectors of this wavefront's share of the row: wavefront w owns the vectors [w * vpw, (w + 1) * vpw)
 // (a contiguous sixteenth of the row, so index order is (wavefront, step, lane, entry)), lane l takes the
 // vectors l, l + 64, ... of that share: every load instruction covers 1 KB of consecutive memory.  Calls
-// f(valid, keys) once per step with the eight 16-bit keys of the lane's vector; the trip count is the same for
-// all lanes, so f may contain wavefront-wide exchanges.  Four loads are in flight per lane.
+// f(valid, plain, keys) once per step with the eight 16-bit keys of the lane's vector (plain: none of them is a
+// zero, an infinity or a NaN); the trip count is the same for all lanes, so f may contain wavefront-wide
+// exchanges.  Four loads are in flight per lane.
 template <typename T, bool HAS_T, typename F>
 __device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, float temp, F &&f) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -895,12 +896,35 @@ __device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, fl
             if (i0 + s * kWave < n_here) {  // wavefront-uniform
                 const uint32_t in[4] = {q[s].x, q[s].y, q[s].z, q[s].w};
                 uint32_t k[8];
+                bool plain = false;  // no zero, infinity or NaN in the vector: two keys per instruction, no selects
+                if constexpr (!HAS_T) {
+                    constexpr uint32_t kAdd = T::kDtype == KA_DTYPE_BF16 ? 0x00800080u : 0x04000400u;
+                    uint32_t special = 0;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    k[2 * c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp);
-                    k[2 * c + 1] = elem_key16<T, HAS_T>(in[c] >> 16, temp);
+                    for (int c = 0; c < 4; ++c) {
+                        const uint32_t mag = in[c] & 0x7fff7fffu;
+                        // bit 15 of a half: set by (mag + kAdd) when its exponent field is all ones; cleared in
+                        // ((mag | 0x8000) - 1) when the half is zero (bit 15 also stops the borrow)
+                        special |= (mag + kAdd) | ~((mag | 0x80008000u) - 0x00010001u);
+                    }
+                    plain = (special & 0x80008000u) == 0;
                 }
-                f(i0 + s * kWave + lane < n_here, k);
+                if (plain) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const uint32_t neg = ((in[c] >> 15) & 0x00010001u) * 0xffffu;  // 0xffff in each negative half
+                        const uint32_t kk = in[c] ^ (neg | 0x80008000u);
+                        k[2 * c] = kk & 0xffffu;
+                        k[2 * c + 1] = kk >> 16;
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        k[2 * c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp);
+                        k[2 * c + 1] = elem_key16<T, HAS_T>(in[c] >> 16, temp);
+                    }
+                }
+                f(i0 + s * kWave + lane < n_here, plain, k);
             }
         }
     }
@@ -959,8 +983,14 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     if (tid == 0) ds.n_inf = 0;
     uint32_t lmax = tail_key;
     uint32_t my_inf = (has_tail && tail_key == kNegInfKey) ? 1u : 0u;
-    for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
-        if (valid) {
+    for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool plain, const uint32_t (&k)[8]) {
+        if (valid && plain) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                atomicAdd(&hist[hist_slot(k[j] >> 1)], (k[j] & 1) ? 0x10000u : 1u);
+                lmax = k[j] > lmax ? k[j] : lmax;
+            }
+        } else if (valid) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 if (k[j] == kNegInfKey) ++my_inf;
@@ -1200,7 +1230,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     {
         uint64_t m = 0;
         uint32_t t = 0;
-        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
+        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool, const uint32_t (&k)[8]) {
             if (valid) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -1266,7 +1296,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         int hstep = 0, step = 0;
         uint64_t hcum = 0;
         uint32_t hrank = 0;
-        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, const uint32_t (&k)[8]) {
+        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool, const uint32_t (&k)[8]) {
             uint64_t m = 0;
             uint32_t t = 0;
             if (valid) {
