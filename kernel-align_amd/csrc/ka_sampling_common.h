@@ -1,0 +1,306 @@
+// Shared pieces of the sampling kernels: order-preserving keys, the integer mass function, exact floor(s * z),
+// temperature rounding, radix level layout, LDS state, block-wide primitives and row traversal.
+#ifndef KA_SAMPLING_COMMON_H
+#define KA_SAMPLING_COMMON_H
+
+#include "ka_common.h"
+
+namespace ka {
+namespace {
+
+constexpr int S_THREADS = 1024;
+constexpr int S_WAVES = S_THREADS / kWave;
+constexpr int BINS = 2048;
+constexpr int FIX_BITS = 40;
+
+// ---------------------------------------------------------------------------
+// Scalar helpers (all exact)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t key_of(float y) {
+    const uint32_t b = __float_as_uint(y);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+// Keys of 16-bit dtypes keep only their significant top bits (a widened bf16 has 16, a widened fp16 19):
+// negative values would otherwise carry ones in the unused low bits, and a key rebuilt from radix digits
+// would not compare equal to the key of the element it came from.
+template <typename T> __device__ __forceinline__ constexpr uint32_t key_mask() {
+    return T::kDtype == KA_DTYPE_BF16 ? 0xffff0000u : (T::kDtype == KA_DTYPE_F16 ? 0xffffe000u : 0xffffffffu);
+}
+template <typename T> __device__ __forceinline__ uint32_t masked_key(float y) { return key_of(y) & key_mask<T>(); }
+template <typename T> __device__ __forceinline__ float value_of(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : (~key & key_mask<T>()));
+}
+
+// W(d) = trunc(2^40 * exp(d)), d <= 0, by a fixed sequence of IEEE double operations: one multiply for the
+// range reduction, a degree-11 Horner evaluation with fused multiply-adds (Taylor coefficients 1/k!), one
+// multiply by a power of two.  Contraction is off in this function, so exactly the operations written here
+// are executed (the CPU statement of the operator performs the same ones, fma() included).  No branches: this
+// runs for up to every entry of a row.
+__device__ __forceinline__ uint64_t weight_fix(float d) {
+#pragma clang fp contract(off)
+    constexpr double C[12] = {0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,
+                              0x1.5555555555555p-3,  0x1.5555555555555p-5,  0x1.1111111111111p-7,
+                              0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16,
+                              0x1.71de3a556c734p-19, 0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26};
+    constexpr double LOG2E = 0x1.71547652b82fep+0, LN2 = 0x1.62e42fefa39efp-1;
+    const double t = double(d) * LOG2E;
+    const double tc = t < -64.0 ? -64.0 : t;  // keeps the conversion below in range; such t give 0 anyway
+    const int n = int(tc - 0.5);
+    const double f = tc - double(n);
+    const double g = f * LN2;
+    double p = C[11];
+#pragma unroll
+    for (int k = 10; k >= 0; --k) p = __builtin_fma(p, g, C[k]);
+    const double scale = __longlong_as_double((long long)(uint64_t(1023 + FIX_BITS + n) << 52));
+    // trunc(p * scale) < 2^42 as an integer: the low mantissa bits of trunc(.) + 2^52
+    const uint64_t w = uint64_t(__double_as_longlong(__builtin_trunc(p * scale) + 0x1p52)) & 0x000fffffffffffffull;
+    const uint64_t special = d > 0.0f ? (uint64_t(1) << FIX_BITS) : 0ull;  // d > 0 cannot occur; NaN -> 0
+    return (d <= 0.0f && !(t < -41.0)) ? w : special;
+}
+
+// log(w / z) for integer masses, in fp64 (w >= 1: an entry of mass 0 is never drawn).
+__device__ __forceinline__ float log_ratio(uint64_t w, uint64_t z) {
+    return float(log(double(w)) - log(double(z)));
+}
+
+// floor(s * z) for an fp32 0 <= s < 1 and z < 2^62.
+__device__ __forceinline__ uint64_t floor_scale(float s, uint64_t z) {
+    const uint32_t b = __float_as_uint(s);
+    const uint32_t e = (b >> 23) & 0xffu, m = b & 0x7fffffu;
+    if (e == 0 && m == 0) return 0;
+    uint64_t mant;
+    int shift;
+    if (e == 0) { mant = m; shift = 149; } else { mant = m | 0x800000u; shift = 150 - int(e); }
+    const uint64_t lo = mant * z, hi = __umul64hi(mant, z);
+    if (shift >= 128) return 0;
+    if (shift >= 64) return hi >> (shift - 64);
+    return (lo >> shift) | (hi << (64 - shift));  // 24 <= shift < 64
+}
+
+// y = x / T rounded to the logits dtype (torch's `logits / temperature`), -0 folded to +0.
+template <typename T> struct Round;
+template <> struct Round<Bf16> {
+    static __device__ __forceinline__ float apply(float q) {
+        uint32_t b = __float_as_uint(q);
+        if ((b & 0x7fffffffu) > 0x7f800000u) return __uint_as_float(((b >> 16) | 0x40u) << 16);
+        b += 0x7fffu + ((b >> 16) & 1u);
+        return __uint_as_float(b & 0xffff0000u);
+    }
+    static constexpr int kLevels = 2;
+};
+template <> struct Round<F16> {
+    static __device__ __forceinline__ float apply(float q) { return float(_Float16(q)); }
+    static constexpr int kLevels = 2;
+};
+template <> struct Round<F32> {
+    static __device__ __forceinline__ float apply(float q) { return q; }
+    static constexpr int kLevels = 3;
+};
+
+// Radix levels, most significant first.  A widened bf16 occupies the top 16 key bits
+// (1 + 8 + 7), a widened fp16 the top 19 (1 + 8 + 10), fp32 all 32.
+template <typename T> __device__ __forceinline__ int level_shift(int level) {
+    if (T::kDtype == KA_DTYPE_BF16) return level == 0 ? 21 : 16;
+    if (T::kDtype == KA_DTYPE_F16) return level == 0 ? 21 : 13;
+    return level == 0 ? 21 : (level == 1 ? 10 : 0);
+}
+template <typename T> __device__ __forceinline__ int level_bits(int level) {
+    if (T::kDtype == KA_DTYPE_BF16) return level == 0 ? 11 : 5;
+    if (T::kDtype == KA_DTYPE_F16) return level == 0 ? 11 : 8;
+    return level == 2 ? 10 : 11;
+}
+
+template <typename T>
+__device__ __forceinline__ uint32_t elem_key(typename T::raw_t raw, float temp, bool has_t) {
+    float y = T::widen(raw);
+    if (has_t) y = Round<T>::apply(y / temp);
+    y = (y == 0.0f) ? 0.0f : y;
+    y = (y != y) ? -__builtin_inff() : y;  // a NaN logit counts as -inf: it is never preferred to a number
+    return masked_key<T>(y);
+}
+
+// ---------------------------------------------------------------------------
+// Block-wide primitives (1024 threads, fixed exchange pattern)
+// ---------------------------------------------------------------------------
+constexpr int CAND_CAP = 1024;  // candidate slots of the top-k fast path (one per thread)
+
+struct Histograms {
+    uint32_t cnt[BINS];
+    uint64_t mass[BINS];
+};
+struct Candidates {            // 24 KB, same footprint as the histograms
+    uint32_t raw[CAND_CAP];    // element bits as loaded (widened to 32 bits)
+    uint32_t idx[CAND_CAP];
+    uint32_t skey[CAND_CAP];   // scaled keys in (key desc, index asc) order; first used for the thread maxima
+    uint32_t sidx[CAND_CAP];
+    uint64_t w[CAND_CAP];      // integer masses in that order
+};
+
+struct DenseScalars {
+    uint64_t wave_u64[S_WAVES];
+    uint32_t wave_u32[S_WAVES];
+    uint64_t seg_mass[S_WAVES + 1];  // dense path: mass of each wavefront's share of the row, and of the ragged tail
+    uint32_t seg_ties[S_WAVES + 1];  // ... and its number of tie-group entries
+    uint64_t z_topk, before_cut, w_cut, pick_w;
+    uint32_t i_topk, n_cut, kcut16, i_last, tie_hi, tie_lo, fail, n_inf;
+    int best_i;
+    int64_t hit;
+};
+
+struct alignas(16) Shared {
+    union {
+        Histograms h;
+        Candidates c;
+    };
+    uint64_t wave_u64[S_WAVES];
+    uint32_t wave_u32[S_WAVES];
+    // broadcast slots
+    uint32_t sel_digit, sel_above, sel_count;
+    uint64_t sel_mass_above, sel_mass;
+    int best_rb;
+    uint32_t max_key;
+    int64_t hit;
+    uint32_t n_cand, pick_a, pick_b;
+    uint64_t pick_z;
+    DenseScalars ds;  // scalars of the resident no-filter path
+};
+
+template <typename V> __device__ __forceinline__ V shfl_up_v(V v, int off) { return __shfl_up(v, off, kWave); }
+
+// Exclusive prefix sum over the block in thread order; *total = block sum.  Contains barriers.
+template <typename V>
+__device__ __forceinline__ V block_excl_scan(V v, V *wave_buf, V *total) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    V inc = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const V t = shfl_up_v(inc, off);
+        if (lane >= off) inc += t;
+    }
+    __syncthreads();  // wave_buf may still be read from a previous call
+    if (lane == kWave - 1) wave_buf[wave] = inc;
+    __syncthreads();
+    V base = 0, sum = 0;
+#pragma unroll
+    for (int w = 0; w < S_WAVES; ++w) {
+        const V x = wave_buf[w];
+        if (w < wave) base += x;
+        sum += x;
+    }
+    *total = sum;
+    return base + inc - v;
+}
+
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, Shared &sh) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t t = __shfl_xor(v, off, kWave);
+        v = t > v ? t : v;
+    }
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) sh.wave_u32[threadIdx.x / kWave] = v;
+    __syncthreads();
+    uint32_t r = sh.wave_u32[0];
+#pragma unroll
+    for (int w = 1; w < S_WAVES; ++w) r = sh.wave_u32[w] > r ? sh.wave_u32[w] : r;
+    return r;
+}
+
+// Finds the bin of sh.h.cnt[0 .. nb) that holds the rank-th largest entry (rank is 1-based, bins are ordered
+// by digit, larger digit = larger keys).  Returns the digit; *above = entries in higher bins, *count =
+// entries in the bin.  Every thread must call it; it contains barriers.
+__device__ __forceinline__ uint32_t select_count_bin(Shared &sh, uint32_t nb, uint32_t rank, uint32_t *above,
+                                                     uint32_t *count) {
+    const int tid = threadIdx.x;
+    // thread t owns the bins 2t and 2t+1 counted from the top
+    const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
+    const uint32_t c0 = rb0 < int(nb) ? sh.h.cnt[nb - 1 - rb0] : 0u;
+    const uint32_t c1 = rb1 < int(nb) ? sh.h.cnt[nb - 1 - rb1] : 0u;
+    uint32_t total;
+    const uint32_t excl = block_excl_scan<uint32_t>(c0 + c1, sh.wave_u32, &total);
+    if (excl < rank && rank <= excl + c0) {
+        sh.sel_digit = nb - 1 - rb0; sh.sel_above = excl; sh.sel_count = c0;
+    } else if (excl + c0 < rank && rank <= excl + c0 + c1) {
+        sh.sel_digit = nb - 1 - rb1; sh.sel_above = excl + c0; sh.sel_count = c1;
+    }
+    __syncthreads();
+    const uint32_t digit = sh.sel_digit;
+    *above = sh.sel_above;
+    *count = sh.sel_count;
+    __syncthreads();
+    return digit;
+}
+
+__device__ __forceinline__ void clear_hist(Shared &sh) {
+    for (int b = threadIdx.x; b < BINS; b += S_THREADS) {
+        sh.h.cnt[b] = 0;
+        sh.h.mass[b] = 0;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row traversal: f(index, raw element) for every element, any order.
+// ---------------------------------------------------------------------------
+template <typename T, int U = 4, typename F>
+__device__ __forceinline__ void for_each_raw(const typename T::raw_t *rp, int vocab, bool vec, F &&f) {
+    constexpr int EPV = T::kPerVec;
+    const int tid = threadIdx.x;
+    if (vec) {
+        const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+        const int nvec = vocab / EPV;
+        int v = tid;
+        for (; v + (U - 1) * S_THREADS < nvec; v += U * S_THREADS) {
+            uint4 q[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) q[u] = vp[v + u * S_THREADS];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[u]);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) f((v + u * S_THREADS) * EPV + j, e[j]);
+            }
+        }
+        for (; v < nvec; v += S_THREADS) {
+            const uint4 q = vp[v];
+            const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) f(v * EPV + j, e[j]);
+        }
+        const int i = nvec * EPV + tid;
+        if (i < vocab) f(i, rp[i]);
+    } else {
+        for (int i = tid; i < vocab; i += S_THREADS) f(i, rp[i]);
+    }
+}
+
+// f(index, key of the scaled element).
+template <typename T, typename F>
+__device__ __forceinline__ void for_each_key(const typename T::raw_t *rp, int vocab, bool vec, float temp,
+                                             bool has_t, F &&f) {
+    for_each_raw<T>(rp, vocab, vec, [&](int i, typename T::raw_t raw) { f(i, elem_key<T>(raw, temp, has_t)); });
+}
+
+// Key of the raw (unscaled) element; the scaling x -> round(x / T) is monotone, so order statistics can be
+// located on these keys and only the few candidates need the division.
+template <typename T> __device__ __forceinline__ uint32_t raw_key(typename T::raw_t raw) {
+    return masked_key<T>(T::widen(raw));
+}
+template <typename T> __device__ __forceinline__ typename T::raw_t raw_of_key(uint32_t key) {
+    const uint32_t bits = __float_as_uint(value_of<T>(key));
+    if (T::kDtype == KA_DTYPE_BF16) return typename T::raw_t(bits >> 16);
+    if (T::kDtype == KA_DTYPE_F16) {
+        union { _Float16 h; uint16_t u; } c;
+        c.h = _Float16(value_of<T>(key));  // exact: the key came from a widened fp16
+        return typename T::raw_t(c.u);
+    }
+    return typename T::raw_t(bits);
+}
+// Distance between neighbouring representable values in key space.
+template <typename T> __device__ __forceinline__ uint32_t key_step() {
+    return T::kDtype == KA_DTYPE_BF16 ? 0x10000u : (T::kDtype == KA_DTYPE_F16 ? 0x2000u : 1u);
+}
+
+}  // namespace
+}  // namespace ka
+
+#endif  // KA_SAMPLING_COMMON_H
