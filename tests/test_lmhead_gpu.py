@@ -74,11 +74,13 @@ def test_rows_are_sliced_to_fit_a_small_workspace_pool(sampler):
     from rl_engine.kernels.pool import PoolExhausted
     from rl_engine.kernels.sampling import SamplerBackend
 
-    hidden, weight, ids = make(1000, 128, 40000, seed=9)                # 3 vocabulary splits: 48 B per row
+    hidden, weight, ids = make(1000, 128, 40000, seed=9)
+    per_row = sampler._lib.ka_lmhead_workspace_bytes(256, 128, 40000) // 256   # 16 B per vocabulary split
+    assert per_row % 16 == 0 and per_row >= 48
     base = sampler.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
-    small = SamplerBackend(pool_bytes=300 * 48).cuda()                   # room for 300 rows -> slices of 256
+    small = SamplerBackend(pool_bytes=300 * per_row).cuda()              # room for 300 rows -> slices of 256
     assert torch.equal(small.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda()), base)
-    tiny = SamplerBackend(pool_bytes=100 * 48).cuda()                    # less than one tile of a long input
+    tiny = SamplerBackend(pool_bytes=100 * per_row).cuda()                    # less than one tile of a long input
     with pytest.raises(PoolExhausted):
         tiny.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
     assert torch.equal(tiny.fused_linear_logp(hidden[:64].cuda(), weight.cuda(), ids[:64].cuda()), base[:64])
