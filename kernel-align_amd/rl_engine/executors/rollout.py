@@ -6,7 +6,9 @@ operators, and ``step`` runs them on a batch of next-token logits.
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Callable, Optional, Tuple
+
+import torch
 
 from rl_engine.kernels.registry import kernel_registry
 from rl_engine.utils.logger import logger
@@ -36,3 +38,33 @@ class RolloutExecutor:
         ids = sample(logits, top_k=self.config.get("top_k"), top_p=self.config.get("top_p"),
                      temperature=self.config.get("temperature", 1.0), uniforms=uniforms)
         return ids, logp(logits, ids)
+
+    def generate(self, next_logits: Callable, prompt_ids, max_new_tokens: int, uniforms=None,
+                 eos_id: Optional[int] = None):
+        """Autoregressive rollout of a group: ``next_logits(ids [B, t]) -> [B, V]`` supplies the logits of
+        the next position; each step samples with the configured filters and records the log-probability
+        of the drawn token under the unfiltered distribution (what the GRPO ratio is built from).
+
+        prompt_ids: int64 [B, T0].  uniforms: optional fp32 [max_new_tokens, B], one draw per row and step.
+        Rows that have produced ``eos_id`` keep emitting it with log-probability 0.  No step synchronises
+        with the host.  Returns (ids [B, T0 + max_new_tokens], logprobs fp32 [B, max_new_tokens]).
+        """
+        if prompt_ids.dim() != 2:
+            raise ValueError("prompt_ids must be [B, T0]")
+        batch, t0 = prompt_ids.shape
+        if uniforms is not None and tuple(uniforms.shape) != (max_new_tokens, batch):
+            raise ValueError(f"uniforms must have shape ({max_new_tokens}, {batch})")
+        ids = torch.empty(batch, t0 + max_new_tokens, dtype=torch.int64, device=prompt_ids.device)
+        ids[:, :t0] = prompt_ids
+        logprobs = torch.zeros(batch, max_new_tokens, dtype=torch.float32, device=prompt_ids.device)
+        done = torch.zeros(batch, dtype=torch.bool, device=prompt_ids.device)
+        for step in range(max_new_tokens):
+            logits = next_logits(ids[:, :t0 + step])
+            tok, lp = self.step(logits, None if uniforms is None else uniforms[step])
+            if eos_id is not None:
+                tok = torch.where(done, torch.full_like(tok, eos_id), tok)
+                lp = torch.where(done, torch.zeros_like(lp), lp)
+                done = done | (tok == eos_id)
+            ids[:, t0 + step] = tok
+            logprobs[:, step] = lp
+        return ids, logprobs

@@ -85,3 +85,13 @@ def test_registry_and_executor():
     assert fn.__name__ == "compute_logp"
     out = RolloutExecutor({"top_k": 50}).execute_rollout()
     assert out == {"status": "success", "kernels": ["HIP_LOGPROB", "HIP_SAMPLING"]}
+
+
+def test_generate_checks_its_arguments_and_never_falls_back_to_the_cpu():
+    executor = RolloutExecutor({"top_k": 4})
+    with pytest.raises(ValueError, match="prompt_ids"):
+        executor.generate(lambda ids: None, torch.zeros(3, dtype=torch.int64), 2)
+    with pytest.raises(ValueError, match="uniforms"):
+        executor.generate(lambda ids: None, torch.zeros(2, 3, dtype=torch.int64), 2, uniforms=torch.zeros(2, 3))
+    with pytest.raises((RuntimeError, ValueError)):     # CPU logits are refused by the operators
+        executor.generate(lambda ids: torch.zeros(2, 16), torch.zeros(2, 3, dtype=torch.int64), 1)

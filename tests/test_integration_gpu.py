@@ -64,3 +64,34 @@ def test_registry_resolves_to_the_hip_operators():
     want = logprob_ref.logprob_ref(logits.cpu(), ids.cpu())
     assert (logp.cpu() - want).abs().max().item() <= 1e-4
     assert kernel_registry.resolve("fused_lm_head_logp").__name__ == "fused_linear_logp"
+
+
+def test_generate_loop_matches_stepwise_oracle():
+    """A toy next-token model (logits = table[last id]) rolled out for 6 steps: every step's ids equal the exact
+    oracle's on the same logits and uniforms, logprobs are those of the unfiltered rows, rows that hit the
+    end-of-sequence id stay there."""
+    from rl_engine.executors.rollout import RolloutExecutor
+
+    gen = torch.Generator().manual_seed(77)
+    vocab, batch, steps, eos = 4096, 8, 6, 5
+    table = (torch.randn(vocab, vocab, generator=gen) * 3.0).bfloat16()
+    table[:, eos] += 4.0                                     # make the end id likely enough to show up
+    prompt = torch.randint(0, vocab, (batch, 3), generator=gen)
+    u = torch.rand(steps, batch, generator=gen)
+    table_gpu = table.cuda()
+    executor = RolloutExecutor({"top_k": 20, "top_p": 0.95, "temperature": 0.8})
+    ids, logp = executor.generate(lambda seq: table_gpu[seq[:, -1]], prompt.cuda(), steps, uniforms=u.cuda(), eos_id=eos)
+    assert ids.shape == (batch, 3 + steps) and torch.equal(ids[:, :3].cpu(), prompt)
+
+    cur, done = prompt[:, -1].clone(), torch.zeros(batch, dtype=torch.bool)
+    for s in range(steps):
+        rows = table[cur]
+        tok = exact.sample(rows, 0.8, 20, 0.95, u[s])
+        lp = logprob_ref.logprob_ref(rows, tok)
+        tok = torch.where(done, torch.full_like(tok, eos), tok)
+        lp = torch.where(done, torch.zeros_like(lp), lp)
+        done |= tok == eos
+        assert torch.equal(ids[:, 3 + s].cpu(), tok), s
+        assert (logp[:, s].cpu() - lp).abs().max().item() <= 1e-4
+        cur = tok
+    assert done.any()
