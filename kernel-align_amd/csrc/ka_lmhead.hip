@@ -2,8 +2,8 @@
 // without materialising the [n_rows, vocab] logits.
 //
 // Tiling (gfx950, wave64, v_mfma_f32_32x32x16_bf16):
-//   * a workgroup of 4 wavefronts owns 256 tokens and walks a range of 256-row
-//     vocabulary tiles; per tile it runs a K loop over the hidden dimension in
+//   * one workgroup of 4 wavefronts per CU walks work items; an item is 256
+//     tokens x a range of 256-row vocabulary tiles; per tile it runs a K loop over the hidden dimension in
 //     slabs of 64 (one cache line per row); the W slab [256 x 64] and the hidden
 //     slab [256 x 64] go from global memory straight into XOR-swizzled LDS
 //     (global_load_lds_dwordx4, no register staging), two stages of 64 KB, one
@@ -30,10 +30,11 @@ constexpr int LM_BN = 256;      // tokens per workgroup
 constexpr int LM_BK = 64;       // hidden slab: one 128-byte line per row
 constexpr int LM_STAGES = 2;    // LDS: the slab in use and the slab in flight
 constexpr int LM_STAGE_ELEMS = (LM_BM + LM_BN) * LM_BK;  // bf16 elements per LDS stage (64 KB)
-constexpr int LM_LDS_BYTES = LM_STAGES * LM_STAGE_ELEMS * 2;
+constexpr int LM_XCH_BYTES = 2 * 4 * 32 * 3 * 4;  // exchange area of the end-of-item fold: [wave_n][tn][32 lanes][3 floats]
+constexpr int LM_LDS_BYTES = LM_STAGES * LM_STAGE_ELEMS * 2 + LM_XCH_BYTES;
 constexpr int LM_THREADS = 256;
-// Vocabulary tiles per split.  8 gives 63 splits at V = 128,256: a single token block already occupies 63 CUs
-// (0.74 ms for 64 rows, against 5.3 ms with 63 tiles per split) and 32,768 rows lose about 1 %.
+// Vocabulary tiles per split (at most).  Short splits let a single token block occupy many CUs: at
+// V = 128,256 (501 tiles, 64 splits of 7 or 8) 64 rows take 0.74 ms, against 5.3 ms with 63 tiles per split.
 constexpr int LM_TILES_PER_SPLIT = 8;
 constexpr int LM_BAR = 24;  // group (of 32 per slab) at which the next slab is waited for; 20..28 measure within 2 %
 constexpr float kLog2e = 1.44269504088896340736f;
@@ -42,6 +43,71 @@ constexpr float kFloor = -1.0e30f;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// The split plan is a function of the vocabulary only, so no row's result depends on the number of rows: a
+// multiple of 8 splits (the width of a super-tile) of nearly equal size, none above LM_TILES_PER_SPLIT tiles.
+__host__ __device__ inline int lm_n_splits(int n_vtiles) {
+    return n_vtiles <= 8 ? n_vtiles : 8 * ((n_vtiles + 8 * LM_TILES_PER_SPLIT - 1) / (8 * LM_TILES_PER_SPLIT));
+}
+// First vocabulary tile of split sp (sp == n_splits: the end).  sp * n_vtiles < 2^31: n_vtiles < 2^17 because the
+// weight matrix is smaller than 4 GiB.
+__host__ __device__ inline int lm_split_begin(int sp, int n_vtiles, int n_splits) {
+    return int(uint32_t(sp) * uint32_t(n_vtiles) / uint32_t(n_splits));
+}
+
+// Work items are (token block, split) pairs, grouped into super-tiles of 4 token blocks x 8 splits.  Item v
+// belongs to the workgroup v % grid; with a grid of 256 that workgroup sits on XCD v % 8 and holds position
+// (v / 8) % 32 of the super-tile that its XCD works on in round v / 256, so the 32 CUs of an XCD run one
+// super-tile side by side and fetch 12 distinct slabs per step instead of 64.
+// Order of the super-tiles: token-block groups are taken eight at a time, one per XCD, and every XCD keeps its
+// four token blocks while it walks all split groups: the hidden rows stay in its L2 / the memory-side cache,
+// and the eight XCDs stream the same W tiles at the same time, so one fetch from HBM serves them all.  (With
+// the token-block group changing at every item each item started on cold hidden rows: 3.5 % slower at
+// 32,768 rows.)  The up to seven token-block groups left over are spread over the XCDs split group by split
+// group, which is also the whole order for fewer than eight groups.
+// Pairs past the ends of the two ranges are not items.
+struct ItemOrder {
+    int sp_groups;  // ceil(n_splits / 8)
+    int full;       // token-block groups handled eight at a time
+    int rest;       // token-block groups left over (0..7)
+    __host__ __device__ ItemOrder(int n_token_blocks, int n_splits) {
+        const int tb_groups = (n_token_blocks + 3) / 4;
+        sp_groups = (n_splits + 7) / 8;
+        full = tb_groups / 8 * 8;
+        rest = tb_groups - full;
+    }
+    __host__ __device__ int rounds_full() const { return full / 8 * sp_groups; }
+    __host__ __device__ int64_t n_virtual() const {  // item indices in use: 256 per round
+        return (int64_t(rounds_full()) + (rest * sp_groups + 7) / 8) * 256;
+    }
+};
+
+__device__ __forceinline__ bool lm_decode(int v, const ItemOrder &order, int n_token_blocks, int n_splits, int &tb,
+                                          int &sp) {
+    const int xcd = v % 8, slot = v / 8;
+    const int round = slot / 32, w = slot % 32;
+    int tg, sg;
+    if (round < order.rounds_full()) {
+        tg = (round / order.sp_groups) * 8 + xcd;
+        sg = round % order.sp_groups;
+    } else {
+        const int q = (round - order.rounds_full()) * 8 + xcd;
+        const int rest = order.rest > 0 ? order.rest : 1;
+        tg = order.full + q % rest;
+        sg = q / rest;
+    }
+    tb = tg * 4 + w / 8;
+    sp = sg * 8 + w % 8;
+    return tb < n_token_blocks && sp < n_splits;
+}
+// The next item of the workgroup that holds item v: indices advance by the grid size.  >= n_virtual: none.
+__device__ __forceinline__ int lm_next_item(int v, int stride, int n_virtual, const ItemOrder &order,
+                                            int n_token_blocks, int n_splits) {
+    int tb, sp;
+    do v += stride;
+    while (v < n_virtual && !lm_decode(v, order, n_token_blocks, n_splits, tb, sp));
+    return v;
+}
 
 struct Partial {
     float m;   // max logit seen (>= kFloor)
@@ -61,7 +127,7 @@ typedef __attribute__((address_space(3))) void lds_void;
 __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
     Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_splits, int n_token_blocks,
-    int n_vtiles) {
+    int n_vtiles, int n_virtual) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [stage][A = W slab | B = hidden slab]
 
     const int tid = threadIdx.x;
@@ -72,36 +138,19 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const int l32 = lane & 31;
     const int lhalf = lane >> 5;
 
-    // (token block, split) pairs are grouped into super-tiles of 4 token blocks x 8 splits; super-tile q goes
-    // to XCD q % 8, whose 32 CUs run its 32 workgroups side by side.  Token-block groups vary fastest, so the
-    // eight XCDs work on the same 8 splits at the same time (one fetch of a W tile from HBM serves them all, and
-    // the W rows of a split group are reused from the memory-side cache by the following token-block groups).
-    // Pairs past the ends do nothing.
-    const int tb_groups = (n_token_blocks + 3) / 4;
-    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
-    const int q = (slot / 32) * 8 + xcd, w = slot % 32;
-    const int tb = (q % tb_groups) * 4 + w / 8;
-    const int sp = (q / tb_groups) * 8 + w % 8;
-    if (tb >= n_token_blocks || sp >= n_splits) return;
-    const int tok0 = tb * LM_BN;
-    const int vt_begin = sp * LM_TILES_PER_SPLIT;
-    const int vt_end = min(n_vtiles, vt_begin + LM_TILES_PER_SPLIT);
+    // A workgroup walks its items v = blockIdx.x, + gridDim.x, ...: with one workgroup per CU nothing is
+    // dispatched between items, and the copies of an item's first slabs are requested while the item before
+    // it is still being multiplied.
+    const ItemOrder order(n_token_blocks, n_splits);
+    const int stride = gridDim.x;
     const int nk = hdim / LM_BK;
+    int v = blockIdx.x, tb, sp;
+    if (!lm_decode(v, order, n_token_blocks, n_splits, tb, sp))
+        v = lm_next_item(v, stride, n_virtual, order, n_token_blocks, n_splits);
+    if (v >= n_virtual) return;
 
-    // This lane's four tokens (one per 32-column block of the wave tile) and their targets.
     float m_run[4], ml2_run[4], s_run[4], xt[4];  // ml2_run = m_run * log2(e), kept so that it is never recomputed
     int target[4];
-#pragma unroll
-    for (int tn = 0; tn < 4; ++tn) {
-        m_run[tn] = kFloor;
-        ml2_run[tn] = kFloor * kLog2e;
-        s_run[tn] = 0.0f;
-        xt[tn] = -__builtin_inff();
-        const int n = tok0 + wave_n * 128 + tn * 32 + l32;
-        int64_t id = -1;
-        if (n < n_rows) id = ids[n];
-        target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
-    }
 
     // Global -> LDS copies.  One global_load_lds_dwordx4 moves 16 B per lane to LDS base + 16 * lane,
     // i.e. one wavefront fills eight consecutive 128-byte rows (eight full cache lines); instruction j of
@@ -109,13 +158,16 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // because the slab is swizzled, the logical chunk (l % 8) ^ swz(row).  Row offsets are 32-bit byte
     // offsets from a wavefront-uniform base (the host checks that both matrices are smaller than 4 GiB).
     const int cp_row = wave * 8 + (lane >> 3);                 // + 32 * j
-    uint32_t hoff[8];
+    uint32_t hoff[8];                                          // hidden rows of the copy cursor's token block
     int cp_chunk[8];                                           // swz depends on bits 1..3 of the row: on j too
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        cp_chunk[j] = (lane & 7) ^ swz(cp_row + 32 * j);
-        hoff[j] = uint32_t(min(tok0 + cp_row + 32 * j, n_rows - 1)) * uint32_t(hdim) * 2u + cp_chunk[j] * 16u;
-    }
+    for (int j = 0; j < 8; ++j) cp_chunk[j] = (lane & 7) ^ swz(cp_row + 32 * j);
+#define LM_SET_HOFF(tok0_)                                                                                    \
+    do {                                                                                                     \
+        _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                        \
+            hoff[j] = uint32_t(min((tok0_) + cp_row + 32 * j, n_rows - 1)) * uint32_t(hdim) * 2u + cp_chunk[j] * 16u; \
+    } while (0)
+    LM_SET_HOFF(tb * LM_BN);
     const int wave_lds = __builtin_amdgcn_readfirstlane(wave) * 512;  // bf16 elements: 8 rows of 64
     const char *const wbytes = reinterpret_cast<const char *>(weight);
     const char *const hbytes = reinterpret_cast<const char *>(hidden);
@@ -133,13 +185,27 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         }                                                                                                    \
     } while (0)
 
-    // Copy cursor: the next slab to request.  Past the last slab of this workgroup it stays on that slab
-    // (redundant copies into the idle stage), so that every step issues the same copies and has no branch.
-    int vt_c = vt_begin, kt_c = 0;
-#define LM_ADVANCE_COPY_CURSOR()                                      \
-    do {                                                              \
-        if (kt_c + 1 < nk) ++kt_c;                                    \
-        else if (vt_c + 1 < vt_end) { ++vt_c; kt_c = 0; }             \
+    // Copy cursor: the next slab to request.  It runs up to two slabs ahead of the MFMAs and crosses from an
+    // item's last slab into the first slab of the workgroup's next item.  Past the last slab of the last item
+    // it stays there (redundant copies into the idle stage), so that every step issues the same copies.
+    int v_c = v, vt_c = lm_split_begin(sp, n_vtiles, n_splits), vt_end_c = lm_split_begin(sp + 1, n_vtiles, n_splits);
+    int kt_c = 0;
+#define LM_ADVANCE_COPY_CURSOR()                                                                              \
+    do {                                                                                                     \
+        if (kt_c + 1 < nk) ++kt_c;                                                                           \
+        else if (vt_c + 1 < vt_end_c) { ++vt_c; kt_c = 0; }                                                   \
+        else {                                                                                               \
+            const int nv_ = lm_next_item(v_c, stride, n_virtual, order, n_token_blocks, n_splits);       \
+            if (nv_ < n_virtual) {                                                                           \
+                int tb_, sp_;                                                                                \
+                lm_decode(nv_, order, n_token_blocks, n_splits, tb_, sp_);                               \
+                v_c = nv_;                                                                                   \
+                vt_c = lm_split_begin(sp_, n_vtiles, n_splits);                                              \
+                vt_end_c = lm_split_begin(sp_ + 1, n_vtiles, n_splits);                                      \
+                kt_c = 0;                                                                                    \
+                LM_SET_HOFF(tb_ * LM_BN);                                                                    \
+            }                                                                                                \
+        }                                                                                                    \
     } while (0)
     // Fragment addresses (bf16 element offsets inside a stage) of this lane at kk = 0; swz() does not depend
     // on kk, so the other k-steps are the same address with the chunk XORed.
@@ -176,6 +242,23 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     }
 
     int stage = 0;
+    for (;;) {  // items of this workgroup; v is a valid item here
+    lm_decode(v, order, n_token_blocks, n_splits, tb, sp);
+    const int tok0 = tb * LM_BN;
+    const int vt_begin = lm_split_begin(sp, n_vtiles, n_splits);
+    const int vt_end = lm_split_begin(sp + 1, n_vtiles, n_splits);
+    // This lane's four tokens (one per 32-column block of the wave tile) and their targets.
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+        m_run[tn] = kFloor;
+        ml2_run[tn] = kFloor * kLog2e;
+        s_run[tn] = 0.0f;
+        xt[tn] = -__builtin_inff();
+        const int n = tok0 + wave_n * 128 + tn * 32 + l32;
+        int64_t id = -1;
+        if (n < n_rows) id = ids[n];
+        target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
+    }
     for (int vt = vt_begin; vt < vt_end; ++vt) {
         f32x16 acc[4][4];
 #pragma unroll
@@ -308,9 +391,9 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         xt[tn] = fmaxf(xt[tn], ox);
     }
     // ---- fold the two vocabulary halves of the tile through LDS (upper half -> lower half) ----
-    float *xch = reinterpret_cast<float *>(lds);  // [wave_n][tn][32][3]
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the trailing (redundant) slab copies may still be writing LDS
-    __syncthreads();
+    // The exchange area lies behind the two stages, which already receive the first slabs of the next item.
+    // One barrier is enough: the area is written again only after the next item's slabs, each with a barrier.
+    float *xch = reinterpret_cast<float *>(lds + LM_STAGES * LM_STAGE_ELEMS);  // [wave_n][tn][32][3]
     if (wave_m == 1 && lhalf == 0) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
@@ -320,7 +403,10 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             p[2] = xt[tn];
         }
     }
-    __syncthreads();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only: the slab copies in flight are not waited for
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
     if (wave_m == 0 && lhalf == 0) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
@@ -339,6 +425,10 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             }
         }
     }
+    v = lm_next_item(v, stride, n_virtual, order, n_token_blocks, n_splits);
+    if (v >= n_virtual) break;
+    }  // items
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the trailing (redundant) slab copies still write LDS
 }
 
 __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict__ partials,
@@ -365,7 +455,7 @@ __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict_
 
 inline int splits_for(int64_t vocab) {
     const int64_t n_vtiles = (vocab + LM_BM - 1) / LM_BM;
-    return int((n_vtiles + LM_TILES_PER_SPLIT - 1) / LM_TILES_PER_SPLIT);
+    return lm_n_splits(int(n_vtiles));
 }
 
 }  // namespace
@@ -400,18 +490,25 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
     const int n_splits = splits_for(vocab);
     const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
-    const int64_t super_tiles = int64_t((n_token_blocks + 3) / 4) * ((n_splits + 7) / 8);
-    const int64_t grid = (super_tiles + 7) / 8 * 8 * 32;  // 32 workgroups per super-tile, super-tiles dealt to 8 XCDs
-    if (grid >= (int64_t(1) << 31)) return fail(KA_ERR_UNSUPPORTED, "lmhead: grid too large");
+    const int64_t n_virtual = ItemOrder(n_token_blocks, n_splits).n_virtual();
+    if (n_virtual >= (int64_t(1) << 30)) return fail(KA_ERR_UNSUPPORTED, "lmhead: too many work items");
+    // One workgroup per CU (a workgroup takes a CU's LDS and registers); each walks its items.  256 workgroups
+    // keep item v on XCD v % 8 and at one position of its super-tiles.
+    int device = 0, cus = 0;
+    hipError_t dev_rc = hipGetDevice(&device);
+    if (dev_rc == hipSuccess) dev_rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    if (dev_rc != hipSuccess) return check_hip(dev_rc, "lmhead: querying the CU count");
+    const int64_t resident = cus >= 256 ? 256 : (cus >= 8 ? cus / 8 * 8 : 8);
+    const int64_t grid = n_virtual < resident ? n_virtual : resident;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     Partial *partials = static_cast<Partial *>(workspace);
     // set on every call rather than once per process: the attribute belongs to the current device
     const hipError_t attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
-    if (attr_rc != hipSuccess) return check_hip(attr_rc, "lmhead: reserving 128 KB of LDS");
+    if (attr_rc != hipSuccess) return check_hip(attr_rc, "lmhead: reserving 131 KB of LDS");
     hipLaunchKernelGGL(lmhead_partials, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                        static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
-                       int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles);
+                       int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
     int rc = check_hip(hipGetLastError(), "lmhead partials launch");
     if (rc != KA_OK) return rc;
     hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids, out,
