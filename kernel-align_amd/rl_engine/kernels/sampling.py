@@ -382,15 +382,24 @@ class SamplerBackend(nn.Module):
         chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
         if chunk < 1:
             raise ValueError("chunk_tokens must be >= 1")
+        if dweight_dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError("dweight_dtype must be torch.float32 or torch.bfloat16")
         dhidden = torch.empty_like(h2)
-        dweight = torch.zeros(w2.shape, dtype=dweight_dtype, device=weight.device)
+        if n_rows == 0:
+            return dhidden.view(hidden.shape), torch.zeros(w2.shape, dtype=dweight_dtype, device=weight.device)
+        dweight = torch.empty(w2.shape, dtype=dweight_dtype, device=weight.device)
+        # bf16 x bf16 GEMMs that write (first chunk) or accumulate into (later chunks) the dweight buffer directly:
+        # no bf16 rounding of a chunk's contribution and no separate add pass over the [V, H] buffer.
+        wide = {"out_dtype": torch.float32} if dweight_dtype == torch.float32 else {}
         for start in range(0, n_rows, chunk):
             stop = min(start + chunk, n_rows)
             logits = torch.matmul(h2[start:stop], w2.t())                       # [n, V] bf16, fp32 accumulation
             logp = self._compute_logp(logits, ids[start:stop])
             self._compute_logp_backward(logits, ids[start:stop], logp, g[start:stop], inplace=True)
             torch.matmul(logits, w2, out=dhidden[start:stop])                   # logits now holds dlogits
-            part = torch.matmul(logits.t(), h2[start:stop])                     # [V, H] bf16
-            dweight.add_(part)
-            del logits, part
+            if start == 0:
+                torch.mm(logits.t(), h2[start:stop], out=dweight, **wide)
+            else:
+                torch.addmm(dweight, logits.t(), h2[start:stop], out=dweight, **wide)
+            del logits
         return dhidden.view(hidden.shape), dweight

@@ -65,7 +65,15 @@ def test_chunked_backward_direct_call_and_shapes(sampler):
     dh_ref, dw_ref = O.lmhead_logprob_backward_ref(hidden.reshape(-1, 192), weight, ids.reshape(-1), grad.reshape(-1))
     assert rel_err(dh.reshape(-1, 192), dh_ref.reshape(-1, 192)) < 2e-2
     assert rel_err(dw, dw_ref) < 2e-2
+    dh16, dw16 = sampler.fused_linear_logp_backward(hidden, weight, ids, grad, chunk_tokens=32,
+                                                    dweight_dtype=torch.bfloat16)
+    assert dw16.dtype == torch.bfloat16 and torch.equal(dh16, dh)
+    assert rel_err(dw16, dw_ref) < 2e-2
+    one_chunk = sampler.fused_linear_logp_backward(hidden, weight, ids, grad, chunk_tokens=80)[1]
+    assert rel_err(one_chunk, dw.double().cpu()) < 1e-3                       # chunking only regroups the fp32 accumulation
     with pytest.raises(ValueError):
         sampler.fused_linear_logp_backward(hidden, weight, ids[:1], grad)
     with pytest.raises(TypeError):
         sampler.fused_linear_logp_backward(hidden.float(), weight, ids, grad)
+    with pytest.raises(TypeError):
+        sampler.fused_linear_logp_backward(hidden, weight, ids, grad, dweight_dtype=torch.float16)
