@@ -32,6 +32,23 @@ def test_small_shapes_against_fp64(sampler, n, h, v):
     assert (got.double() - want).abs().max().item() <= TOL
 
 
+@pytest.mark.parametrize("n,h,v", [(9000, 64, 5000),      # 36 token blocks: eight groups walked XCD-resident + one left over;
+                                                            # one hidden slab per tile, so the copy cursor crosses items at once
+                                   (8300, 128, 70000),     # 274 vocabulary tiles = 40 splits (5 split groups), two slabs per tile
+                                   (16640, 64, 300)])      # 65 token blocks, two tiles = two one-tile splits
+def test_many_token_blocks_walk_several_items_per_workgroup(sampler, n, h, v):
+    """More (token block, split) items than CUs: every workgroup walks several items and its copy pipeline runs
+    across their boundaries.  Checked against the CPU oracle, and bit for bit against a short call on the
+    first rows (the split plan depends on the vocabulary only)."""
+    hidden, weight, ids = make(n, h, v, seed=n + v, w_scale=0.2)
+    hg, wg, ig = hidden.cuda(), weight.cuda(), ids.cuda()
+    got = sampler.fused_linear_logp(hg, wg, ig)
+    want = O.lmhead_logprob_ref(hidden, weight, ids, dtype=torch.float32 if v > 10000 else torch.float64)
+    assert (got.cpu().double() - want.double()).abs().max().item() <= TOL
+    assert torch.equal(got[:300], sampler.fused_linear_logp(hg[:300], wg, ig[:300]))
+    assert torch.equal(got[-517:], sampler.fused_linear_logp(hg[-517:], wg, ig[-517:]))
+
+
 def test_llama_shape_slice(sampler):
     hidden, weight, ids = make(384, 4096, 128256, seed=0)
     got = sampler.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda()).cpu()
