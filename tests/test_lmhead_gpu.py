@@ -60,6 +60,22 @@ def test_llama_shape_slice(sampler):
     assert (got - unfused).abs().max().item() <= TOL
 
 
+def test_full_baseline_shape(sampler):
+    """hidden [32768, 4096] x W [128256, 4096] (generated on the device): 64 scattered rows against the fp32 CPU
+    oracle, and two row ranges bit for bit against calls of their own."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+    hidden = torch.randn(32768, 4096, generator=g, device="cuda").bfloat16()
+    weight = (torch.randn(128256, 4096, generator=g, device="cuda") * 0.02).bfloat16()
+    ids = torch.randint(0, 128256, (32768,), generator=g, device="cuda")
+    got = sampler.fused_linear_logp(hidden, weight, ids)
+    assert torch.isfinite(got).all()
+    pick = torch.randperm(32768, generator=torch.Generator().manual_seed(1))[:64].sort().values
+    want = O.lmhead_logprob_ref(hidden[pick.cuda()].cpu(), weight.cpu(), ids[pick.cuda()].cpu(), dtype=torch.float32)
+    assert (got[pick.cuda()].cpu() - want).abs().max().item() <= TOL
+    for lo, hi in ((0, 256), (20000, 20777)):
+        assert torch.equal(got[lo:hi], sampler.fused_linear_logp(hidden[lo:hi], weight, ids[lo:hi]))
+
+
 def test_leading_dims_and_invalid_ids(sampler):
     hidden, weight, ids = make(96, 128, 3000, seed=3, w_scale=0.2)
     ids[5], ids[6] = 3000, -2
