@@ -69,6 +69,41 @@ def test_sampling_argument_checks():
     assert ex(0, p, 2, 128, 128, 0.0, p, -1, p, 9.0, p, p, p, None, None, 0, None) == _hip.KA_ERR_HIP
 
 
+def test_lmhead_argument_checks_and_workspace_size():
+    lib = _hip.load()
+    p = ctypes.c_void_p(4096)
+    call = lib.ka_lmhead_logprob_bf16
+    ws = lib.ka_lmhead_workspace_bytes
+    # 16 B per row and vocabulary split; the split count depends on the vocabulary only
+    assert ws(0, 4096, 128256) == 0
+    assert ws(1, 4096, 128256) == 16 * 64 and ws(32768, 4096, 128256) == 32768 * 16 * 64
+    assert ws(5, 64, 256) == 5 * 16 and ws(5, 64, 257) == 5 * 32 and ws(5, 64, 8 * 256) == 5 * 16 * 8
+    assert ws(5, 64, 9 * 256) == 5 * 16 * 8 and ws(5, 64, 65 * 256) == 5 * 16 * 16
+    assert ws(7, 64, 128256) == ws(7, 8192, 128256)
+    assert call(None, None, None, None, 0, 4096, 128256, None, 0, None) == _hip.KA_OK             # no rows
+    assert call(None, p, p, p, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG
+    assert call(p, p, p, p, -1, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG
+    assert call(p, p, p, p, 4, 100, 128256, p, 1 << 20, None) == _hip.KA_ERR_UNSUPPORTED           # H % 64
+    assert call(ctypes.c_void_p(4100), p, p, p, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_UNSUPPORTED
+    assert call(p, p, p, p, 4, 4096, 1 << 20, p, 1 << 30, None) == _hip.KA_ERR_UNSUPPORTED         # W of 8 GiB
+    assert call(p, p, p, p, 4, 4096, 128256, None, 0, None) == _hip.KA_ERR_WORKSPACE
+    assert call(p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
+    assert b"workspace" in lib.ka_last_error()
+
+
+def test_grpo_and_backward_argument_checks():
+    lib = _hip.load()
+    p = ctypes.c_void_p(4096)
+    g = lib.ka_grpo_token_terms
+    assert g(None, None, None, None, 0, 0.2, 0.2, 0.0, None, None, None, None) == _hip.KA_OK
+    assert g(None, None, None, p, 8, 0.2, 0.2, 0.0, p, p, p, None) == _hip.KA_ERR_BAD_ARG       # logp_new missing
+    assert g(p, None, None, p, -3, 0.2, 0.2, 0.0, p, p, p, None) == _hip.KA_ERR_BAD_ARG
+    b = lib.ka_logprob_backward_bf16
+    assert b.argtypes is not None
+    assert lib.ka_sample_mass_fixed(None, 0, None, None) == _hip.KA_OK
+    assert lib.ka_sample_mass_fixed(None, 4, p, None) == _hip.KA_ERR_BAD_ARG
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setenv(_hip.ENV_LIB, str(tmp_path / "nope.so"))
     monkeypatch.setattr(_hip, "_lib", None)
