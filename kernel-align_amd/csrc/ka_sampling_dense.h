@@ -315,12 +315,48 @@ __device__ __forceinline__ int hist_slot(int word) {
     return word ^ ((word >> 4) & 0x1c);  // chunk index (bits 2..4) ^= bits 1..3 of the block index (bits 6..8)
 }
 
+// The eight 16-bit keys of one 16-byte vector.  Returns true if none of the values is a zero, an infinity or a
+// NaN (only looked for without a temperature): such a vector converts two keys per instruction, with no selects.
+template <typename T, bool HAS_T>
+__device__ __forceinline__ bool vector_keys(const uint4 &q, float temp, uint32_t (&k)[8]) {
+    const uint32_t in[4] = {q.x, q.y, q.z, q.w};
+    bool plain = false;
+    if constexpr (!HAS_T) {
+        constexpr uint32_t kAdd = T::kDtype == KA_DTYPE_BF16 ? 0x00800080u : 0x04000400u;
+        uint32_t special = 0;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t mag = in[c] & 0x7fff7fffu;
+            // bit 15 of a half: set by (mag + kAdd) when its exponent field is all ones; cleared in
+            // ((mag | 0x8000) - 1) when the half is zero (bit 15 also stops the borrow)
+            special |= (mag + kAdd) | ~((mag | 0x80008000u) - 0x00010001u);
+        }
+        plain = (special & 0x80008000u) == 0;
+    }
+    if (plain) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t neg = ((in[c] >> 15) & 0x00010001u) * 0xffffu;  // 0xffff in each negative half
+            const uint32_t kk = in[c] ^ (neg | 0x80008000u);
+            k[2 * c] = kk & 0xffffu;
+            k[2 * c + 1] = kk >> 16;
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            k[2 * c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp);
+            k[2 * c + 1] = elem_key16<T, HAS_T>(in[c] >> 16, temp);
+        }
+    }
+    return plain;
+}
+
 // Walks the vectors of this wavefront's share of the row: wavefront w owns the vectors [w * vpw, (w + 1) * vpw)
 // (a contiguous sixteenth of the row, so index order is (wavefront, step, lane, entry)), lane l takes the
 // vectors l, l + 64, ... of that share: every load instruction covers 1 KB of consecutive memory.  Calls
-// f(valid, plain, keys) once per step with the eight 16-bit keys of the lane's vector (plain: none of them is a
-// zero, an infinity or a NaN); the trip count is the same for all lanes, so f may contain wavefront-wide
-// exchanges.  Four loads are in flight per lane.
+// f(valid, plain, keys) once per step with the eight 16-bit keys of the lane's vector (plain: see vector_keys);
+// the trip count is the same for all lanes, so f may contain wavefront-wide exchanges.  Four loads are in
+// flight per lane.
 template <typename T, bool HAS_T, typename F>
 __device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, float temp, F &&f) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -335,36 +371,8 @@ __device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, fl
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             if (i0 + s * kWave < n_here) {  // wavefront-uniform
-                const uint32_t in[4] = {q[s].x, q[s].y, q[s].z, q[s].w};
                 uint32_t k[8];
-                bool plain = false;  // no zero, infinity or NaN in the vector: two keys per instruction, no selects
-                if constexpr (!HAS_T) {
-                    constexpr uint32_t kAdd = T::kDtype == KA_DTYPE_BF16 ? 0x00800080u : 0x04000400u;
-                    uint32_t special = 0;
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const uint32_t mag = in[c] & 0x7fff7fffu;
-                        // bit 15 of a half: set by (mag + kAdd) when its exponent field is all ones; cleared in
-                        // ((mag | 0x8000) - 1) when the half is zero (bit 15 also stops the borrow)
-                        special |= (mag + kAdd) | ~((mag | 0x80008000u) - 0x00010001u);
-                    }
-                    plain = (special & 0x80008000u) == 0;
-                }
-                if (plain) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const uint32_t neg = ((in[c] >> 15) & 0x00010001u) * 0xffffu;  // 0xffff in each negative half
-                        const uint32_t kk = in[c] ^ (neg | 0x80008000u);
-                        k[2 * c] = kk & 0xffffu;
-                        k[2 * c + 1] = kk >> 16;
-                    }
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        k[2 * c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp);
-                        k[2 * c + 1] = elem_key16<T, HAS_T>(in[c] >> 16, temp);
-                    }
-                }
+                const bool plain = vector_keys<T, HAS_T>(q[s], temp, k);
                 f(i0 + s * kWave + lane < n_here, plain, k);
             }
         }
@@ -727,19 +735,21 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
             seen += t;
         }
     }
-    // 7c. inside the segment: the step, the lane, the entry (one wavefront works, the others wait at the barrier)
-    if (seg == wave) {
-        uint64_t cum = acc;
-        uint32_t rank = ties_before;
-        bool found = false;
-        uint32_t hk[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // this lane's keys in the step that holds tau
-        bool hvalid = false;
-        int hstep = 0, step = 0;
-        uint64_t hcum = 0;
-        uint32_t hrank = 0;
-        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool, const uint32_t (&k)[8]) {
-            uint64_t m = 0;
-            uint32_t t = 0;
+    // 7c. inside the segment (a wavefront's share: at most S_WAVES steps of 64 vectors): every wavefront sums one
+    //     step, then the wavefront whose step holds tau finds the lane and the entry
+    if (seg >= 0 && seg < S_WAVES) {  // the same for the whole block
+        const int sv0 = seg * vpw;
+        const int n_seg = nvec - sv0 < vpw ? nvec - sv0 : vpw;
+        const int n_steps = (n_seg + kWave - 1) / kWave;
+        const int lane = tid & (kWave - 1);
+        const int idx = wave * kWave + lane;
+        const bool valid = idx < n_seg;
+        uint32_t k[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        uint64_t m = 0;
+        uint32_t t = 0;
+        if (wave < n_steps) {
+            const uint4 q = valid ? (reinterpret_cast<const uint4 *>(rp) + sv0)[idx] : make_uint4(0, 0, 0, 0);
+            vector_keys<T, false>(q, 1.0f, k);
             if (valid) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -747,46 +757,57 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
                     t += is_tie(k[j]) ? 1u : 0u;
                 }
             }
-            const uint64_t ms = wave_sum_u64(m);
-            const uint32_t ts = wave_sum_u32(t);
-            const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
-            const uint64_t total = ms + uint64_t(ts < room ? ts : room) * w_tie;
-            if (!found && tau < cum + total) {  // wavefront-uniform
-                found = true;
-                hstep = step;
-                hcum = cum;
-                hrank = rank;
-                hvalid = valid;
+        }
+        const uint64_t ms = wave_sum_u64(m);
+        const uint32_t ts = wave_sum_u32(t);
+        if (lane == 0) {
+            ds.wave_u64[wave] = ms;
+            ds.wave_u32[wave] = ts;
+        }
+        __syncthreads();
+        uint64_t cum = acc, hcum = 0;
+        uint32_t rank = ties_before, hrank = 0;
+        int hstep = -1;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) hk[j] = k[j];
+        for (int st = 0; st < S_WAVES; ++st) {
+            if (st < n_steps) {
+                const uint32_t st_ties = ds.wave_u32[st];
+                const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
+                const uint64_t total = ds.wave_u64[st] + uint64_t(st_ties < room ? st_ties : room) * w_tie;
+                if (hstep < 0 && tau < cum + total) {
+                    hstep = st;
+                    hcum = cum;
+                    hrank = rank;
+                }
+                cum += total;
+                rank += st_ties;
             }
-            cum += total;
-            rank += ts;
-            ++step;
-        });
-        // lanes of that step in order: tie ranks first, then masses
-        uint32_t lt = 0;
+        }
+        if (wave == hstep) {
+            // lanes of that step in order: tie ranks first, then masses
+            uint32_t lt = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) lt += (hvalid && is_tie(hk[j])) ? 1u : 0u;
-        uint32_t rk = hrank + wave_excl_scan<uint32_t>(lt);
-        const uint32_t rk0 = rk;
-        uint64_t lm = 0;
+            for (int j = 0; j < 8; ++j) lt += (valid && is_tie(k[j])) ? 1u : 0u;
+            uint32_t rk = hrank + wave_excl_scan<uint32_t>(lt);
+            const uint32_t rk0 = rk;
+            uint64_t lm = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            if (hvalid) lm += is_tie(hk[j]) ? ((rk++ < r_cut) ? w_tie : 0ull) : mass(hk[j]);
-        const uint64_t before = hcum + wave_excl_scan<uint64_t>(lm);
-        if (before <= tau && tau < before + lm) {
-            uint64_t c2 = before;
-            uint32_t r2 = rk0;
-            bool done = false;
+            for (int j = 0; j < 8; ++j)
+                if (valid) lm += is_tie(k[j]) ? ((rk++ < r_cut) ? w_tie : 0ull) : mass(k[j]);
+            const uint64_t before = hcum + wave_excl_scan<uint64_t>(lm);
+            if (before <= tau && tau < before + lm) {
+                uint64_t c2 = before;
+                uint32_t r2 = rk0;
+                bool done = false;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint64_t wj = is_tie(hk[j]) ? ((r2++ < r_cut) ? w_tie : 0ull) : mass(hk[j]);
-                c2 += wj;
-                if (!done && c2 > tau) {
-                    done = true;
-                    ds.hit = (v0 + hstep * kWave + (tid & (kWave - 1))) * 8 + j;
-                    ds.pick_w = wj;
+                for (int j = 0; j < 8; ++j) {
+                    const uint64_t wj = is_tie(k[j]) ? ((r2++ < r_cut) ? w_tie : 0ull) : mass(k[j]);
+                    c2 += wj;
+                    if (!done && c2 > tau) {
+                        done = true;
+                        ds.hit = (sv0 + hstep * kWave + lane) * 8 + j;
+                        ds.pick_w = wj;
+                    }
                 }
             }
         }
