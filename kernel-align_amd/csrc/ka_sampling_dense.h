@@ -315,38 +315,44 @@ __device__ __forceinline__ int hist_slot(int word) {
     return word ^ ((word >> 4) & 0x1c);  // chunk index (bits 2..4) ^= bits 1..3 of the block index (bits 6..8)
 }
 
-// The eight 16-bit keys of one 16-byte vector.  Returns true if none of the values is a zero, an infinity or a
-// NaN (only looked for without a temperature): such a vector converts two keys per instruction, with no selects.
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+
+// Key j (0..7) of a vector whose keys are packed two per dword (entry 2c in the low half of dword c).
+__device__ __forceinline__ uint32_t key_at(const uint32_t (&kk)[4], int j) {
+    return (j & 1) ? kk[j >> 1] >> 16 : kk[j >> 1] & 0xffffu;
+}
+
+// The eight 16-bit keys of one 16-byte vector, two per dword.  Returns true if none of the values is a zero, an
+// infinity or a NaN (only looked for without a temperature): such a vector is converted with packed 16-bit
+// instructions, three per two keys, and no selects.
 template <typename T, bool HAS_T>
-__device__ __forceinline__ bool vector_keys(const uint4 &q, float temp, uint32_t (&k)[8]) {
+__device__ __forceinline__ bool vector_keys(const uint4 &q, float temp, uint32_t (&kk)[4]) {
     const uint32_t in[4] = {q.x, q.y, q.z, q.w};
     bool plain = false;
     if constexpr (!HAS_T) {
-        constexpr uint32_t kAdd = T::kDtype == KA_DTYPE_BF16 ? 0x00800080u : 0x04000400u;
-        uint32_t special = 0;
+        // magnitude - 1 (wrapping in 16 bits) is 0xffff for a zero and at least kInf - 1 for an infinity or a NaN
+        constexpr uint32_t kInf = T::kDtype == KA_DTYPE_BF16 ? 0x7f80u : 0x7c00u;
+        u16x2 worst = {0, 0};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const uint32_t mag = in[c] & 0x7fff7fffu;
-            // bit 15 of a half: set by (mag + kAdd) when its exponent field is all ones; cleared in
-            // ((mag | 0x8000) - 1) when the half is zero (bit 15 also stops the borrow)
-            special |= (mag + kAdd) | ~((mag | 0x80008000u) - 0x00010001u);
+            const u16x2 mag = __builtin_bit_cast(u16x2, in[c] & 0x7fff7fffu);
+            worst = __builtin_elementwise_max(worst, mag - u16x2{1, 1});
         }
-        plain = (special & 0x80008000u) == 0;
+        const uint32_t w = __builtin_bit_cast(uint32_t, worst);
+        const uint32_t m = (w & 0xffffu) > (w >> 16) ? (w & 0xffffu) : (w >> 16);
+        plain = m < kInf - 1u;
     }
     if (plain) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const uint32_t neg = ((in[c] >> 15) & 0x00010001u) * 0xffffu;  // 0xffff in each negative half
-            const uint32_t kk = in[c] ^ (neg | 0x80008000u);
-            k[2 * c] = kk & 0xffffu;
-            k[2 * c + 1] = kk >> 16;
+            const uint32_t neg = __builtin_bit_cast(uint32_t, __builtin_bit_cast(i16x2, in[c]) >> 15);  // 0xffff in each negative half
+            kk[c] = in[c] ^ (neg | 0x80008000u);
         }
     } else {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            k[2 * c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp);
-            k[2 * c + 1] = elem_key16<T, HAS_T>(in[c] >> 16, temp);
-        }
+        for (int c = 0; c < 4; ++c)
+            kk[c] = elem_key16<T, HAS_T>(in[c] & 0xffffu, temp) | (elem_key16<T, HAS_T>(in[c] >> 16, temp) << 16);
     }
     return plain;
 }
@@ -354,7 +360,8 @@ __device__ __forceinline__ bool vector_keys(const uint4 &q, float temp, uint32_t
 // Walks the vectors of this wavefront's share of the row: wavefront w owns the vectors [w * vpw, (w + 1) * vpw)
 // (a contiguous sixteenth of the row, so index order is (wavefront, step, lane, entry)), lane l takes the
 // vectors l, l + 64, ... of that share: every load instruction covers 1 KB of consecutive memory.  Calls
-// f(valid, plain, keys) once per step with the eight 16-bit keys of the lane's vector (plain: see vector_keys);
+// f(valid, plain, keys) once per step with the eight 16-bit keys of the lane's vector, packed two per dword
+// (plain: see vector_keys);
 // the trip count is the same for all lanes, so f may contain wavefront-wide exchanges.  Four loads are in
 // flight per lane.
 template <typename T, bool HAS_T, typename F>
@@ -371,9 +378,9 @@ __device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, fl
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             if (i0 + s * kWave < n_here) {  // wavefront-uniform
-                uint32_t k[8];
-                const bool plain = vector_keys<T, HAS_T>(q[s], temp, k);
-                f(i0 + s * kWave + lane < n_here, plain, k);
+                uint32_t kk[4];
+                const bool plain = vector_keys<T, HAS_T>(q[s], temp, kk);
+                f(i0 + s * kWave + lane < n_here, plain, kk);
             }
         }
     }
@@ -432,22 +439,36 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     if (tid == 0) ds.n_inf = 0;
     uint32_t lmax = tail_key;
     uint32_t my_inf = (has_tail && tail_key == kNegInfKey) ? 1u : 0u;
-    for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool plain, const uint32_t (&k)[8]) {
+    u16x2 lmax2 = {0, 0};
+    unsigned char *const hist_bytes = reinterpret_cast<unsigned char *>(hist);
+    for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool plain, const uint32_t (&kk)[4]) {
         if (valid && plain) {
+            // two keys per dword all the way: histogram word of a key = key >> 1, swizzled as in hist_slot(); its
+            // counter is the low half for an even key, the high half for an odd one
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                atomicAdd(&hist[hist_slot(k[j] >> 1)], (k[j] & 1) ? 0x10000u : 1u);
-                lmax = k[j] > lmax ? k[j] : lmax;
+            for (int c = 0; c < 4; ++c) {
+                lmax2 = __builtin_elementwise_max(lmax2, __builtin_bit_cast(u16x2, kk[c]));
+                const uint32_t w2 = (kk[c] >> 1) & 0x7fff7fffu;
+                const uint32_t slot2 = w2 ^ ((w2 >> 4) & 0x001c001cu);
+                atomicAdd(reinterpret_cast<uint32_t *>(hist_bytes + ((slot2 << 2) & 0x3fffcu)), (kk[c] & 1u) * 0xffffu + 1u);
+                atomicAdd(reinterpret_cast<uint32_t *>(hist_bytes + ((slot2 >> 14) & 0x3fffcu)),
+                          ((kk[c] >> 16) & 1u) * 0xffffu + 1u);
             }
         } else if (valid) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                if (k[j] == kNegInfKey) ++my_inf;
-                else atomicAdd(&hist[hist_slot(k[j] >> 1)], (k[j] & 1) ? 0x10000u : 1u);
-                lmax = k[j] > lmax ? k[j] : lmax;
+                const uint32_t k = key_at(kk, j);
+                if (k == kNegInfKey) ++my_inf;
+                else atomicAdd(&hist[hist_slot(k >> 1)], (k & 1) ? 0x10000u : 1u);
+                lmax = k > lmax ? k : lmax;
             }
         }
     });
+    {
+        const uint32_t m2 = __builtin_bit_cast(uint32_t, lmax2);
+        lmax = (m2 & 0xffffu) > lmax ? (m2 & 0xffffu) : lmax;
+        lmax = (m2 >> 16) > lmax ? (m2 >> 16) : lmax;
+    }
     if (has_tail && tail_key != kNegInfKey) atomicAdd(&hist[hist_slot(tail_key >> 1)], (tail_key & 1) ? 0x10000u : 1u);
     my_inf = wave_sum_u32(my_inf);
     __syncthreads();  // ds.n_inf is zero
@@ -679,12 +700,12 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     {
         uint64_t m = 0;
         uint32_t t = 0;
-        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool, const uint32_t (&k)[8]) {
+        for_wave_vectors<T, false>(vp, n_here, 1.0f, [&](bool valid, bool, const uint32_t (&kk)[4]) {
             if (valid) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    m += mass(k[j]);
-                    t += is_tie(k[j]) ? 1u : 0u;
+                    m += mass(key_at(kk, j));
+                    t += is_tie(key_at(kk, j)) ? 1u : 0u;
                 }
             }
         });
@@ -744,18 +765,20 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         const int lane = tid & (kWave - 1);
         const int idx = wave * kWave + lane;
         const bool valid = idx < n_seg;
-        uint32_t k[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        uint32_t kk[4] = {0, 0, 0, 0}, k[8];
         uint64_t m = 0;
         uint32_t t = 0;
         if (wave < n_steps) {
             const uint4 q = valid ? (reinterpret_cast<const uint4 *>(rp) + sv0)[idx] : make_uint4(0, 0, 0, 0);
-            vector_keys<T, false>(q, 1.0f, k);
-            if (valid) {
+            vector_keys<T, false>(q, 1.0f, kk);
+        }
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    m += mass(k[j]);
-                    t += is_tie(k[j]) ? 1u : 0u;
-                }
+        for (int j = 0; j < 8; ++j) k[j] = key_at(kk, j);
+        if (wave < n_steps && valid) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                m += mass(k[j]);
+                t += is_tie(k[j]) ? 1u : 0u;
             }
         }
         const uint64_t ms = wave_sum_u64(m);
