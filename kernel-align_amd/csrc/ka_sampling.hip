@@ -323,17 +323,18 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                     ka_sample_workspace_bytes(batch, vocab));
     const bool aligned = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * T::kBytes) % 16 == 0);
     const bool no_fast = force_radix_path();
-    // The dense-histogram path needs 157 KB of LDS (one workgroup per CU).  It serves top-p without top-k and
-    // top_k > 1024 on 16-bit rows that fit in registers; with per-row parameters any row may need it.
+    // The dense-histogram path needs 157 KB of LDS (one workgroup per CU).  It serves top-p without top-k,
+    // top_k > 1024 and no filter at all on aligned 16-bit rows; with per-row parameters any row may need it.
     bool dense = false;
-    if (T::kBytes == 2 && aligned && !no_fast && vocab / 8 <= RES_VECS * S_THREADS) {
+    if (T::kBytes == 2 && aligned && !no_fast) {
         const bool per_row = prm.top_k_rows != nullptr || prm.top_p_rows != nullptr;
         const bool k_on = prm.top_k > 0 && prm.top_k < vocab;
         // (no filter at all: the histogram path for bf16; an fp16 row has too many distinct values for its list and
         //  takes the register-resident no-filter path of the small-LDS kernel)
         const bool no_filter = !k_on && !(prm.top_p < 1.0f);
+        const bool fits_registers = vocab / 8 <= RES_VECS * S_THREADS;  // what the other kernel's no-filter path takes
         dense = per_row || (k_on && prm.top_k > S_THREADS) || (!k_on && !no_filter) ||
-                (no_filter && T::kDtype == KA_DTYPE_BF16);
+                (no_filter && (T::kDtype == KA_DTYPE_BF16 || !fits_registers));
     }
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const typename T::raw_t *lp = static_cast<const typename T::raw_t *>(logits);

@@ -8,7 +8,8 @@ namespace ka {
 namespace {
 
 // ---------------------------------------------------------------------------
-// Paths for 16-bit dtypes (bf16, fp16), rows of at most 131,072 entries, 16-byte aligned.
+// Paths for 16-bit dtypes (bf16, fp16), 16-byte aligned rows (the register-resident no-filter path: at most
+// 131,072 entries; the dense path streams the row and takes any length).
 // Since a 16-bit dtype has only 65,536 values, an entry's integer mass is a function of its 16-bit key.
 //
 //   no filter   : the row is read once into registers (16 x uint4 per lane, a contiguous run of entries per
@@ -407,7 +408,7 @@ template <typename T, bool HAS_T, bool ALL_SURVIVE>
 __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename T::raw_t *rp, int vocab, bool vec,
                                              float temp, bool use_k, int top_k, bool use_p, float top_p, float u,
                                              int64_t *out_slot, float *lp_slot) {
-    if (!resident_ok<T>(vocab, vec)) return false;
+    if (!vec || T::kBytes != 2) return false;  // rows of any length: nothing of the row is kept
     uint32_t *hist = reinterpret_cast<uint32_t *>(lds);
     uint32_t *list = hist + D_WORDS;                                   // (key << 16) | count, descending keys
     uint64_t *table = reinterpret_cast<uint64_t *>(list);              // later: mass of key kcut16 + i
@@ -756,83 +757,92 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
             seen += t;
         }
     }
-    // 7c. inside the segment (a wavefront's share: at most S_WAVES steps of 64 vectors): every wavefront sums one
-    //     step, then the wavefront whose step holds tau finds the lane and the entry
+    // 7c. inside the segment (a wavefront's share of the row, in steps of 64 vectors): every wavefront sums one step,
+    //     then the wavefront whose step holds tau finds the lane and the entry.  A share of more than S_WAVES steps
+    //     (rows above 131,072 entries) takes further rounds of S_WAVES steps.
     if (seg >= 0 && seg < S_WAVES) {  // the same for the whole block
         const int sv0 = seg * vpw;
         const int n_seg = nvec - sv0 < vpw ? nvec - sv0 : vpw;
         const int n_steps = (n_seg + kWave - 1) / kWave;
         const int lane = tid & (kWave - 1);
-        const int idx = wave * kWave + lane;
-        const bool valid = idx < n_seg;
-        uint32_t kk[4] = {0, 0, 0, 0}, k[8];
-        uint64_t m = 0;
-        uint32_t t = 0;
-        if (wave < n_steps) {
-            const uint4 q = valid ? (reinterpret_cast<const uint4 *>(rp) + sv0)[idx] : make_uint4(0, 0, 0, 0);
-            vector_keys<T, false>(q, 1.0f, kk);
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) k[j] = key_at(kk, j);
-        if (wave < n_steps && valid) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                m += mass(k[j]);
-                t += is_tie(k[j]) ? 1u : 0u;
+        uint64_t cum = acc;
+        uint32_t rank = ties_before;
+        for (int st0 = 0; st0 < n_steps; st0 += S_WAVES) {  // block-uniform trip count and exit
+            const int idx = (st0 + wave) * kWave + lane;
+            const bool valid = idx < n_seg;
+            uint32_t kk[4] = {0, 0, 0, 0}, k[8];
+            uint64_t m = 0;
+            uint32_t t = 0;
+            if (st0 + wave < n_steps) {
+                const uint4 q = valid ? (reinterpret_cast<const uint4 *>(rp) + sv0)[idx] : make_uint4(0, 0, 0, 0);
+                vector_keys<T, false>(q, 1.0f, kk);
             }
-        }
-        const uint64_t ms = wave_sum_u64(m);
-        const uint32_t ts = wave_sum_u32(t);
-        if (lane == 0) {
-            ds.wave_u64[wave] = ms;
-            ds.wave_u32[wave] = ts;
-        }
-        __syncthreads();
-        uint64_t cum = acc, hcum = 0;
-        uint32_t rank = ties_before, hrank = 0;
-        int hstep = -1;
 #pragma unroll
-        for (int st = 0; st < S_WAVES; ++st) {
-            if (st < n_steps) {
-                const uint32_t st_ties = ds.wave_u32[st];
-                const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
-                const uint64_t total = ds.wave_u64[st] + uint64_t(st_ties < room ? st_ties : room) * w_tie;
-                if (hstep < 0 && tau < cum + total) {
-                    hstep = st;
-                    hcum = cum;
-                    hrank = rank;
-                }
-                cum += total;
-                rank += st_ties;
-            }
-        }
-        if (wave == hstep) {
-            // lanes of that step in order: tie ranks first, then masses
-            uint32_t lt = 0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) lt += (valid && is_tie(k[j])) ? 1u : 0u;
-            uint32_t rk = hrank + wave_excl_scan<uint32_t>(lt);
-            const uint32_t rk0 = rk;
-            uint64_t lm = 0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (valid) lm += is_tie(k[j]) ? ((rk++ < r_cut) ? w_tie : 0ull) : mass(k[j]);
-            const uint64_t before = hcum + wave_excl_scan<uint64_t>(lm);
-            if (before <= tau && tau < before + lm) {
-                uint64_t c2 = before;
-                uint32_t r2 = rk0;
-                bool done = false;
+            for (int j = 0; j < 8; ++j) k[j] = key_at(kk, j);
+            if (valid) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const uint64_t wj = is_tie(k[j]) ? ((r2++ < r_cut) ? w_tie : 0ull) : mass(k[j]);
-                    c2 += wj;
-                    if (!done && c2 > tau) {
-                        done = true;
-                        ds.hit = (sv0 + hstep * kWave + lane) * 8 + j;
-                        ds.pick_w = wj;
-                    }
+                    m += mass(k[j]);
+                    t += is_tie(k[j]) ? 1u : 0u;
                 }
             }
+            const uint64_t ms = wave_sum_u64(m);
+            const uint32_t ts = wave_sum_u32(t);
+            if (lane == 0) {
+                ds.wave_u64[wave] = ms;
+                ds.wave_u32[wave] = ts;
+            }
+            __syncthreads();
+            uint64_t hcum = 0;
+            uint32_t hrank = 0;
+            int hstep = -1;
+#pragma unroll
+            for (int st = 0; st < S_WAVES; ++st) {
+                if (st0 + st < n_steps) {
+                    const uint32_t st_ties = ds.wave_u32[st];
+                    const uint32_t room = rank < r_cut ? r_cut - rank : 0u;
+                    const uint64_t total = ds.wave_u64[st] + uint64_t(st_ties < room ? st_ties : room) * w_tie;
+                    if (hstep < 0 && tau < cum + total) {
+                        hstep = st;
+                        hcum = cum;
+                        hrank = rank;
+                    }
+                    cum += total;
+                    rank += st_ties;
+                }
+            }
+            if (hstep >= 0) {
+                if (wave == hstep) {
+                    // lanes of that step in order: tie ranks first, then masses
+                    uint32_t lt = 0;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) lt += (valid && is_tie(k[j])) ? 1u : 0u;
+                    uint32_t rk = hrank + wave_excl_scan<uint32_t>(lt);
+                    const uint32_t rk0 = rk;
+                    uint64_t lm = 0;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (valid) lm += is_tie(k[j]) ? ((rk++ < r_cut) ? w_tie : 0ull) : mass(k[j]);
+                    const uint64_t before = hcum + wave_excl_scan<uint64_t>(lm);
+                    if (before <= tau && tau < before + lm) {
+                        uint64_t c2 = before;
+                        uint32_t r2 = rk0;
+                        bool done = false;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const uint64_t wj = is_tie(k[j]) ? ((r2++ < r_cut) ? w_tie : 0ull) : mass(k[j]);
+                            c2 += wj;
+                            if (!done && c2 > tau) {
+                                done = true;
+                                ds.hit = (sv0 + idx) * 8 + j;
+                                ds.pick_w = wj;
+                            }
+                        }
+                    }
+                }
+                break;
+            }
+            __syncthreads();  // the per-step totals are overwritten by the next round
         }
     } else if (seg == S_WAVES && wave == 0) {
         const bool tie = has_tail && is_tie(tail_key);

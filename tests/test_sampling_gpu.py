@@ -92,6 +92,20 @@ def test_ragged_vocab(sampler, vocab):
     check_exact(sampler, logits, u, None, 0.9, 1.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("vocab", [131080, 151936, 262144 + 1032])
+def test_rows_longer_than_the_register_file(sampler, dtype, vocab):
+    """Rows above 131,072 entries stay on the histogram path (a wavefront's share of the row is searched in
+    rounds of sixteen steps); every filter combination against the exact oracle, draws spread over the row."""
+    g = torch.Generator().manual_seed(vocab)
+    logits = (torch.randn(8, vocab, generator=g) * (3 if dtype == torch.bfloat16 else 1.5)).to(dtype)
+    logits[3, vocab // 2:] = float("-inf")                    # masked second half
+    logits[4] = logits[4, 0]                                   # one value: the draw is uniform over the row
+    u = torch.tensor([0.0, 0.03, 0.31, 0.5, 0.77, 0.93, 0.999, 0.9999999])
+    for k, p, t in [(None, None, 1.0), (None, 0.9, 0.7), (None, 0.999, 1.3), (2000, 0.9, 0.7), (50, 0.9, 0.7)]:
+        check_exact(sampler, logits, u, k, p, t)
+
+
 def test_unaligned_and_strided_rows(sampler):
     g = torch.Generator().manual_seed(23)
     big = (torch.randn(12, 4104, generator=g) * 3).bfloat16()
