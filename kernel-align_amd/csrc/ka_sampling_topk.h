@@ -33,33 +33,42 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     constexpr int RES_VECS = 16;
     const int nvec = vocab / EPV;
     const bool resident = vec && T::kDtype == KA_DTYPE_BF16 && nvec <= RES_VECS * S_THREADS;
-    // A longer or wider row (fp32: up to 131,072 entries) does not fit in registers, but the maximum of each of
-    // the lane's vectors does: the collection pass then re-reads only the few vectors that hold a candidate.
+    // A longer or wider row does not fit in registers, but 32 maxima per lane do: slot r keeps the maximum of the
+    // lane's vectors tid + (g * 32 + r) * 1024, g = 0 .. trk_rounds - 1, and the collection pass re-reads only the
+    // slots that hold a candidate.  One vector per slot covers an fp32 row of 131,072 entries and a 16-bit row of
+    // 262,144; longer fp32 rows take up to four vectors per slot (for the 16-bit dtypes the count stays a
+    // compile-time 1, which keeps their kernels as they are).
     constexpr int TRK_VECS = 32;
-    const bool tracked = vec && !resident && nvec <= TRK_VECS * S_THREADS;
+    const int trk_need = (nvec + TRK_VECS * S_THREADS - 1) / (TRK_VECS * S_THREADS);
+    const int trk_rounds = T::kBytes == 4 ? trk_need : 1;
+    const bool tracked = vec && !resident && trk_need <= (T::kBytes == 4 ? 4 : 1);
     uint4 held[RES_VECS];
     float vmaxs[TRK_VECS];
     float lmaxf = -__builtin_inff();
     if (tracked) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+#pragma unroll 1
+        for (int round = 0; round < trk_rounds; ++round) {
+            const int base = tid + round * TRK_VECS * S_THREADS;
 #pragma unroll
-        for (int g = 0; g < TRK_VECS / 8; ++g) {
-            uint4 q[8];
+            for (int g = 0; g < TRK_VECS / 8; ++g) {
+                uint4 q[8];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int v = tid + (g * 8 + s) * S_THREADS;
-                q[s] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
-            }
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                float vm = -__builtin_inff();
-                if (tid + (g * 8 + s) * S_THREADS < nvec) {
-                    const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[s]);
-#pragma unroll
-                    for (int j = 0; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
+                for (int s = 0; s < 8; ++s) {
+                    const int v = base + (g * 8 + s) * S_THREADS;
+                    q[s] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
                 }
-                vmaxs[g * 8 + s] = vm;
-                lmaxf = fmaxf(lmaxf, vm);
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    float vm = -__builtin_inff();
+                    if (base + (g * 8 + s) * S_THREADS < nvec) {
+                        const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[s]);
+#pragma unroll
+                        for (int j = 0; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
+                    }
+                    vmaxs[g * 8 + s] = round == 0 ? vm : fmaxf(vmaxs[g * 8 + s], vm);
+                    lmaxf = fmaxf(lmaxf, vm);
+                }
             }
         }
         const int i = nvec * EPV + tid;  // ragged tail of the row
@@ -153,12 +162,16 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll
         for (int r = 0; r < TRK_VECS; ++r) {
-            if (vmaxs[r] >= boundf) {  // rare: about top_k vectors of the whole row hold a candidate
-                const int v = tid + r * S_THREADS;
-                const uint4 q = vp[v];
-                const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+            if (vmaxs[r] >= boundf) {  // rare: about top_k slots of the whole row hold a candidate
+                for (int round = 0; round < trk_rounds; ++round) {
+                    const int v = tid + (round * TRK_VECS + r) * S_THREADS;
+                    if (v < nvec) {
+                        const uint4 q = vp[v];
+                        const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
 #pragma unroll
-                for (int j = 0; j < EPV; ++j) collect(v * EPV + j, e[j]);
+                        for (int j = 0; j < EPV; ++j) collect(v * EPV + j, e[j]);
+                    }
+                }
             }
         }
         const int i = nvec * EPV + tid;

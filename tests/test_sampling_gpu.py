@@ -106,6 +106,19 @@ def test_rows_longer_than_the_register_file(sampler, dtype, vocab):
         check_exact(sampler, logits, u, k, p, t)
 
 
+@pytest.mark.parametrize("dtype,vocab", [(torch.float32, 151936), (torch.float32, 300004), (torch.bfloat16, 600008),
+                                         (torch.float16, 262144)])
+def test_top_k_on_rows_longer_than_the_tracked_maxima(sampler, dtype, vocab):
+    """The top-k fast path keeps 32 maxima per lane; above 32,768 vectors a maximum covers several vectors."""
+    g = torch.Generator().manual_seed(vocab + 1)
+    logits = (torch.randn(8, vocab, generator=g) * 2.5).to(dtype)
+    logits[2, : vocab - 5] = float("-inf")                    # fewer entries than top_k above -inf
+    logits[5, vocab // 3] = 30.0
+    u = torch.tensor([0.0, 0.11, 0.35, 0.5, 0.62, 0.8, 0.97, 0.9999999])
+    for k, p, t in [(50, 0.9, 0.7), (1, None, 1.0), (1000, 0.95, 1.0), (7, None, 1.5)]:
+        check_exact(sampler, logits, u, k, p, t)
+
+
 def test_unaligned_and_strided_rows(sampler):
     g = torch.Generator().manual_seed(23)
     big = (torch.randn(12, 4104, generator=g) * 3).bfloat16()
