@@ -21,6 +21,7 @@
 #include "ka_sampling_common.h"
 #include "ka_sampling_dense.h"
 #include "ka_sampling_topk.h"
+#include "ka_sampling_draw.h"
 
 namespace ka {
 namespace {
@@ -61,7 +62,11 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                                                          int no_fast) {
     constexpr int EPV = T::kPerVec;
     constexpr int LEVELS = Round<T>::kLevels;
-    unsigned char *const lds = lds_base<DENSE>();
+    // For fp32 rows the second variant is the radix path alone, with the draw done by shares of the row; the host
+    // launches it for the filter combinations that the top-k fast path does not serve.  (Kept apart because the
+    // register allocation of the fast path suffers when the code behind it grows.)
+    constexpr bool RADIX_ONLY = DENSE && T::kBytes == 4;
+    unsigned char *const lds = lds_base<DENSE && T::kBytes == 2>();
     Shared &sh = *reinterpret_cast<Shared *>(lds);
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.x;
@@ -83,8 +88,10 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (!(u >= 0.0f)) u = 0.0f;
     if (u >= 1.0f) u = __uint_as_float(0x3f7fffffu);
 
-    if (use_k && top_k <= S_THREADS && !no_fast) {
-        if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot)) return;
+    if (!RADIX_ONLY && use_k && top_k <= S_THREADS && !no_fast) {
+        if constexpr (!RADIX_ONLY) {
+            if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot)) return;
+        }
         __syncthreads();
     } else if (!no_fast) {
         if constexpr (DENSE && T::kBytes == 2) {
@@ -146,23 +153,26 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     }
 
     // ---- masses of the survivors of top-k: total, and level-0 histogram for top-p ---------
-    clear_hist(sh);
-    __syncthreads();
-    uint64_t zpart = 0;
-    for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
-        if (key >= kstar) {
-            const float y = value_of<T>(key);
-            const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
-            zpart += w;
-            if (use_p) {
-                atomicAdd(reinterpret_cast<unsigned long long *>(&sh.h.mass[key >> 21]), (unsigned long long)w);
-                atomicAdd(&sh.h.cnt[key >> 21], 1u);
+    // (the draw by shares finds the total itself: without top-p this pass is not needed)
+    uint64_t z_topk = 0;
+    if (!(RADIX_ONLY && vec && !use_p)) {
+        clear_hist(sh);
+        __syncthreads();
+        uint64_t zpart = 0;
+        for_each_key<T>(rp, vocab, vec, temp, has_t, [&](int, uint32_t key) {
+            if (key >= kstar) {
+                const float y = value_of<T>(key);
+                const uint64_t w = weight_fix(key == kmax ? 0.0f : y - vmax);
+                zpart += w;
+                if (use_p) {
+                    atomicAdd(reinterpret_cast<unsigned long long *>(&sh.h.mass[key >> 21]), (unsigned long long)w);
+                    atomicAdd(&sh.h.cnt[key >> 21], 1u);
+                }
             }
-        }
-    });
-    uint64_t z_topk;
-    block_excl_scan<uint64_t>(zpart, sh.wave_u64, &z_topk);
-    __syncthreads();
+        });
+        block_excl_scan<uint64_t>(zpart, sh.wave_u64, &z_topk);
+        __syncthreads();
+    }
 
     // ---- top-p: descent to the lowest key whose first entry is still kept ------------------
     uint32_t kcut = kstar;            // survivors: key > kcut, or key == kcut with tie rank < r_cut
@@ -229,6 +239,12 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     }
 
     // ---- draw: first survivor, in index order, whose inclusive mass exceeds floor(u * Z) ----
+    if constexpr (RADIX_ONLY) {
+        if (vec) {
+            draw_by_shares<T>(sh.ds, rp, vocab, temp, has_t, kmax, vmax, kcut, r_cut, u, out + row, lp_slot);
+            return;
+        }
+    }
     const uint64_t tau = floor_scale(u, z_kept);
     const bool track_ties = r_cut != 0xffffffffu;
     if (tid == 0) sh.hit = -1;
@@ -338,6 +354,17 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
     }
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const typename T::raw_t *lp = static_cast<const typename T::raw_t *>(logits);
+    if constexpr (T::kBytes == 4) {
+        // fp32 rows outside the top-k fast path (no filter, top-p alone, top_k > 1024): the radix path with the draw
+        // done by shares of the row
+        const bool per_row = prm.top_k_rows != nullptr || prm.top_p_rows != nullptr;
+        const bool k_fast = prm.top_k > 0 && prm.top_k < vocab && prm.top_k <= S_THREADS;
+        if (aligned && !per_row && !k_fast) {
+            hipLaunchKernelGGL((sample_rows<T, true>), dim3(unsigned(batch)), dim3(S_THREADS), 0, stream, lp, int(vocab),
+                               row_stride, prm, 1, no_fast ? 1 : 0);
+            return check_hip(hipGetLastError(), "sample launch");
+        }
+    }
     if constexpr (T::kBytes == 2) {
       if (dense) {
         const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(sample_rows<T, true>),
