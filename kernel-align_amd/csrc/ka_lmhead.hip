@@ -49,10 +49,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 __host__ __device__ inline int lm_n_splits(int n_vtiles) {
     return n_vtiles <= 8 ? n_vtiles : 8 * ((n_vtiles + 8 * LM_TILES_PER_SPLIT - 1) / (8 * LM_TILES_PER_SPLIT));
 }
-// First vocabulary tile of split sp (sp == n_splits: the end).  sp * n_vtiles < 2^31: n_vtiles < 2^17 because the
-// weight matrix is smaller than 4 GiB.
+// First vocabulary tile of split sp (sp == n_splits: the end).
 __host__ __device__ inline int lm_split_begin(int sp, int n_vtiles, int n_splits) {
-    return int(uint32_t(sp) * uint32_t(n_vtiles) / uint32_t(n_splits));
+    return int(uint64_t(sp) * uint64_t(n_vtiles) / uint64_t(n_splits));
 }
 
 // Work items are (token block, split) pairs, grouped into super-tiles of 4 token blocks x 8 splits.  Item v
@@ -124,6 +123,9 @@ __device__ __forceinline__ int swz(int row) { return (row >> 1) & 7; }
 
 typedef __attribute__((address_space(3))) void lds_void;
 
+// WIDE: a matrix of 4 GiB or more.  Hidden rows are then addressed relative to the cursor's token block and W rows by
+// 64-bit offsets; the ordinary kernel keeps 32-bit offsets from the two base pointers, which is 1 - 2 % faster.
+template <bool WIDE>
 __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
     Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_splits, int n_token_blocks,
@@ -155,8 +157,9 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // Global -> LDS copies.  One global_load_lds_dwordx4 moves 16 B per lane to LDS base + 16 * lane,
     // i.e. one wavefront fills eight consecutive 128-byte rows (eight full cache lines); instruction j of
     // wavefront w covers rows (4j + w) * 8 .. + 7.  Lane l therefore fetches row (4j + w) * 8 + l / 8 and,
-    // because the slab is swizzled, the logical chunk (l % 8) ^ swz(row).  Row offsets are 32-bit byte
-    // offsets from a wavefront-uniform base (the host checks that both matrices are smaller than 4 GiB).
+    // because the slab is swizzled, the logical chunk (l % 8) ^ swz(row).  Row offsets are 32-bit byte offsets
+    // from a wavefront-uniform base: the matrix itself, or with WIDE the cursor's token block (hidden) and a
+    // 64-bit product (W).
     const int cp_row = wave * 8 + (lane >> 3);                 // + 32 * j
     uint32_t hoff[8];                                          // hidden rows of the copy cursor's token block
     int cp_chunk[8];                                           // swz depends on bits 1..3 of the row: on j too
@@ -165,12 +168,14 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
 #define LM_SET_HOFF(tok0_)                                                                                    \
     do {                                                                                                     \
         _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                        \
-            hoff[j] = uint32_t(min((tok0_) + cp_row + 32 * j, n_rows - 1)) * uint32_t(hdim) * 2u + cp_chunk[j] * 16u; \
+            hoff[j] = uint32_t(min(cp_row + 32 * j + (WIDE ? 0 : (tok0_)), n_rows - 1 - (WIDE ? (tok0_) : 0))) * row_bytes + cp_chunk[j] * 16u; \
+        if (WIDE) hbase = reinterpret_cast<const char *>(hidden) + size_t(tok0_) * row_bytes;                \
     } while (0)
+    const uint32_t row_bytes = uint32_t(hdim) * 2u;
+    const char *hbase = reinterpret_cast<const char *>(hidden);  // WIDE: first hidden row of the cursor's token block
     LM_SET_HOFF(tb * LM_BN);
     const int wave_lds = __builtin_amdgcn_readfirstlane(wave) * 512;  // bf16 elements: 8 rows of 64
     const char *const wbytes = reinterpret_cast<const char *>(weight);
-    const char *const hbytes = reinterpret_cast<const char *>(hidden);
 
     // Requests copy c (0..15: W rows for even c, hidden rows for odd c) of slab (vt_, kt_) into stage stage_.
 #define LM_ISSUE_ONE(c_, vt_, kt_, stage_)                                                                   \
@@ -178,10 +183,16 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         const size_t kb_ = size_t(kt_) * (LM_BK * 2);                                                        \
         uint16_t *sa_ = lds + (stage_) * LM_STAGE_ELEMS + wave_lds + ((c_) >> 1) * 2048;                      \
         if (((c_) & 1) == 0) {                                                                               \
-            const uint32_t woff_ = uint32_t(min((vt_) * LM_BM + cp_row + 32 * ((c_) >> 1), vocab - 1)) * uint32_t(hdim) * 2u + cp_chunk[(c_) >> 1] * 16u; \
-            __builtin_amdgcn_global_load_lds(wbytes + kb_ + woff_, (lds_void *)sa_, 16, 0, 0);               \
+            const uint32_t wrow_ = uint32_t(min((vt_) * LM_BM + cp_row + 32 * ((c_) >> 1), vocab - 1));        \
+            if constexpr (WIDE) {                                                                            \
+                const uint64_t woff_ = uint64_t(wrow_) * row_bytes + uint32_t(cp_chunk[(c_) >> 1] * 16);      \
+                __builtin_amdgcn_global_load_lds(wbytes + kb_ + woff_, (lds_void *)sa_, 16, 0, 0);           \
+            } else {                                                                                         \
+                const uint32_t woff_ = wrow_ * row_bytes + cp_chunk[(c_) >> 1] * 16u;                        \
+                __builtin_amdgcn_global_load_lds(wbytes + kb_ + woff_, (lds_void *)sa_, 16, 0, 0);           \
+            }                                                                                                \
         } else {                                                                                             \
-            __builtin_amdgcn_global_load_lds(hbytes + kb_ + hoff[(c_) >> 1], (lds_void *)(sa_ + LM_BM * LM_BK), 16, 0, 0); \
+            __builtin_amdgcn_global_load_lds(hbase + kb_ + hoff[(c_) >> 1], (lds_void *)(sa_ + LM_BM * LM_BK), 16, 0, 0); \
         }                                                                                                    \
     } while (0)
 
@@ -482,8 +493,6 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
         return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden and weight must be 16-byte aligned");
     if (n_rows >= (int64_t(1) << 31) || vocab >= (int64_t(1) << 31) || hidden_dim >= (int64_t(1) << 31))
         return fail(KA_ERR_UNSUPPORTED, "lmhead: a dimension does not fit 31 bits");
-    if (n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32))
-        return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden or weight matrix of 4 GiB or more (32-bit row offsets)");
     const size_t need = ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab);
     if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
         return fail(KA_ERR_WORKSPACE, "lmhead: workspace of %zu B (16-byte aligned) needed, got %zu B", need, workspace_bytes);
@@ -502,13 +511,20 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     const int64_t grid = n_virtual < resident ? n_virtual : resident;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     Partial *partials = static_cast<Partial *>(workspace);
+    const bool wide = n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32);
+    const void *kernel = wide ? reinterpret_cast<const void *>(lmhead_partials<true>)
+                              : reinterpret_cast<const void *>(lmhead_partials<false>);
     // set on every call rather than once per process: the attribute belongs to the current device
-    const hipError_t attr_rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
+    const hipError_t attr_rc = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
     if (attr_rc != hipSuccess) return check_hip(attr_rc, "lmhead: reserving 131 KB of LDS");
-    hipLaunchKernelGGL(lmhead_partials, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
-                       static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
-                       int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
+    if (wide)
+        hipLaunchKernelGGL(lmhead_partials<true>, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
+                           static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
+                           int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
+    else
+        hipLaunchKernelGGL(lmhead_partials<false>, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
+                           static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
+                           int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
     int rc = check_hip(hipGetLastError(), "lmhead partials launch");
     if (rc != KA_OK) return rc;
     hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids, out,

@@ -85,7 +85,7 @@ def test_lmhead_argument_checks_and_workspace_size():
     assert call(p, p, p, p, -1, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG
     assert call(p, p, p, p, 4, 100, 128256, p, 1 << 20, None) == _hip.KA_ERR_UNSUPPORTED           # H % 64
     assert call(ctypes.c_void_p(4100), p, p, p, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_UNSUPPORTED
-    assert call(p, p, p, p, 4, 4096, 1 << 20, p, 1 << 30, None) == _hip.KA_ERR_UNSUPPORTED         # W of 8 GiB
+    assert call(p, p, p, p, 4, 4096, 1 << 31, p, 1 << 40, None) == _hip.KA_ERR_UNSUPPORTED         # vocab of 2^31
     assert call(p, p, p, p, 4, 4096, 128256, None, 0, None) == _hip.KA_ERR_WORKSPACE
     assert call(p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
     assert b"workspace" in lib.ka_last_error()

@@ -76,6 +76,26 @@ def test_full_baseline_shape(sampler):
         assert torch.equal(got[lo:hi], sampler.fused_linear_logp(hidden[lo:hi], weight, ids[lo:hi]))
 
 
+def test_weight_matrix_above_4_gib(sampler):
+    """W [300000, 8192] bf16 is 4.9 GB: row offsets beyond 32 bits.  Rows with targets in the last part of the
+    vocabulary against the fp32 CPU oracle, all rows against the unfused path on the GPU."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    vocab, hdim, n = 300000, 8192, 320
+    weight = torch.empty(vocab, hdim, dtype=torch.bfloat16, device="cuda")
+    for lo in range(0, vocab, 50000):                                    # generated in pieces: no 9.8 GB fp32 temporary
+        weight[lo:lo + 50000] = (torch.randn(50000, hdim, generator=g, device="cuda") * 0.02).bfloat16()
+    hidden = torch.randn(n, hdim, generator=g, device="cuda").bfloat16()
+    ids = torch.randint(0, vocab, (n,), generator=g, device="cuda")
+    ids[:8] = torch.tensor([vocab - 1, vocab - 2, 262144, 262143, 280000, 299999 - 256, 0, 131072], device="cuda")
+    got = sampler.fused_linear_logp(hidden, weight, ids)
+    logits = torch.cat([torch.nn.functional.linear(hidden.float(), weight[lo:lo + 50000].float())
+                        for lo in range(0, vocab, 50000)], dim=1)
+    unfused = sampler.compute_logp(logits, ids)
+    assert (got - unfused).abs().max().item() <= TOL
+    want = O.lmhead_logprob_ref(hidden[:8].cpu(), weight.cpu(), ids[:8].cpu(), dtype=torch.float32)
+    assert (got[:8].cpu() - want).abs().max().item() <= TOL
+
+
 def test_leading_dims_and_invalid_ids(sampler):
     hidden, weight, ids = make(96, 128, 3000, seed=3, w_scale=0.2)
     ids[5], ids[6] = 3000, -2
