@@ -16,14 +16,15 @@ namespace {
 //                 lane) and every entry is replaced by the key of its scaled value; one pass evaluates every
 //                 entry's mass, one block-wide prefix sum of the lane totals finds the lane that holds the
 //                 draw, which then finds the vector and the entry.
-//   dense path  : (top-p without top-k, or top_k > 1024) a count histogram over all 65,536 raw keys in LDS
+//   dense path  : (no filter on bf16 rows, top-p without top-k, or top_k > 1024) a count histogram over all 65,536 raw keys in LDS
 //                 (16-bit counters, two per word) is filled by one streaming pass and compacted into a list
 //                 of the occupied keys in descending order; temperature and masses are applied once per
 //                 occupied key (a few thousand instead of 128 K; runs of keys that scale to one value form
 //                 one tie group); prefix sums over the list give the top-k key, Z, the top-p cut and the
 //                 surviving mass; the masses of the surviving keys go into a table indexed by
-//                 key - lowest surviving key, and the draw streams the row twice more (from L2 / MALL):
-//                 per-wavefront masses first, then the step, lane and entry inside one wavefront's share.
+//                 key - lowest surviving key, and the draw streams the row once more (from L2 / MALL) for the
+//                 mass of every wavefront's share, then re-reads the share that holds the target, one 64-vector
+//                 step per wavefront, to find the step, the lane and the entry.
 // Both return false (having written no output) when a row does not fit (a counter overflow, too many occupied
 // keys, survivors spanning too many keys, a temperature that folds more than 64 values into one); the radix
 // path then runs.  All integer decisions are the same function of the row as in the radix path.
