@@ -49,6 +49,23 @@ def test_many_token_blocks_walk_several_items_per_workgroup(sampler, n, h, v):
     assert torch.equal(got[-517:], sampler.fused_linear_logp(hg[-517:], wg, ig[-517:]))
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_randomised_shapes(sampler, seed):
+    """Random row counts (1 .. 40 token blocks and a ragged last one), hidden sizes and vocabularies (1 .. 160
+    tiles with a ragged last one): every (token block, split) item order and split plan against the oracle."""
+    rng = torch.Generator().manual_seed(1000 + seed)
+    for _ in range(5):
+        h = int(torch.randint(1, 5, (1,), generator=rng)) * 64
+        v = int(torch.randint(1, 40000, (1,), generator=rng))
+        n = int(torch.randint(1, 10000, (1,), generator=rng))
+        while n * v * h > 2.5e10:                              # keep the CPU oracle within a second or two
+            n = n // 2 + 1
+        hidden, weight, ids = make(n, h, v, seed=n + v + h, w_scale=0.15)
+        got = sampler.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda()).cpu()
+        want = O.lmhead_logprob_ref(hidden, weight, ids, dtype=torch.float32)
+        assert (got - want).abs().max().item() <= TOL, (n, h, v)
+
+
 def test_llama_shape_slice(sampler):
     hidden, weight, ids = make(384, 4096, 128256, seed=0)
     got = sampler.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda()).cpu()
