@@ -169,6 +169,11 @@ int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, void *hip_str
  * hidden: bf16 [n_rows, hidden_dim] row-major; weight: bf16 [vocab, hidden_dim]
  * row-major (the nn.Linear.weight layout).  bf16 MFMA with fp32 accumulation;
  * logit tiles stay in registers and feed an online max / log-sum-exp.
+ * hidden_dim must be a multiple of 64 and both matrices 16-byte aligned; the
+ * workspace (16 bytes per row and vocabulary split, as the query reports) must
+ * be 16-byte aligned.  A row's result does not depend on n_rows.  An id outside
+ * [0, vocab) gives NaN for its row.  The kernel is launched as one workgroup
+ * per CU, each walking its share of the work.
  * No counterpart in the reference; the nearest behaviour is
  * compute_logp(lm_head(hidden)) (rl_engine/kernels/sampling.py:92-112).
  */
