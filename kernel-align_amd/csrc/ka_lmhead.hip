@@ -54,24 +54,29 @@ __host__ __device__ inline int lm_split_begin(int sp, int n_vtiles, int n_splits
     return int(uint64_t(sp) * uint64_t(n_vtiles) / uint64_t(n_splits));
 }
 
-// Work items are (token block, split) pairs, grouped into super-tiles of 4 token blocks x 8 splits.  Item v
+// Work items are (token block, split) pairs, grouped into super-tiles of tbw token blocks x 32 / tbw splits.  Item v
 // belongs to the workgroup v % grid; with a grid of 256 that workgroup sits on XCD v % 8 and holds position
 // (v / 8) % 32 of the super-tile that its XCD works on in round v / 256, so the 32 CUs of an XCD run one
 // super-tile side by side and fetch 12 distinct slabs per step instead of 64.
 // Order of the super-tiles: token-block groups are taken eight at a time, one per XCD, and every XCD keeps its
-// four token blocks while it walks all split groups: the hidden rows stay in its L2 / the memory-side cache,
+// token blocks while it walks all split groups: the hidden rows stay in its L2 / the memory-side cache,
 // and the eight XCDs stream the same W tiles at the same time, so one fetch from HBM serves them all.  (With
 // the token-block group changing at every item each item started on cold hidden rows: 3.5 % slower at
 // 32,768 rows.)  The up to seven token-block groups left over are spread over the XCDs split group by split
 // group, which is also the whole order for fewer than eight groups.
-// Pairs past the ends of the two ranges are not items.
+// Shape of the super-tile: 8 token blocks x 4 splits when that fills the XCDs eight groups at a time (64 token
+// blocks or more: every XCD then passes over W half as often; 2 - 3 % faster at 32,768 rows), else 4 x 8.
+// Neither the order nor the shape changes any result.  Pairs past the ends of the two ranges are not items.
 struct ItemOrder {
-    int sp_groups;  // ceil(n_splits / 8)
+    int tbw, spw;   // token blocks and splits of a super-tile (tbw * spw == 32)
+    int sp_groups;  // ceil(n_splits / spw)
     int full;       // token-block groups handled eight at a time
     int rest;       // token-block groups left over (0..7)
     __host__ __device__ ItemOrder(int n_token_blocks, int n_splits) {
-        const int tb_groups = (n_token_blocks + 3) / 4;
-        sp_groups = (n_splits + 7) / 8;
+        tbw = n_token_blocks >= 64 ? 8 : 4;
+        spw = 32 / tbw;
+        const int tb_groups = (n_token_blocks + tbw - 1) / tbw;
+        sp_groups = (n_splits + spw - 1) / spw;
         full = tb_groups / 8 * 8;
         rest = tb_groups - full;
     }
@@ -95,8 +100,8 @@ __device__ __forceinline__ bool lm_decode(int v, const ItemOrder &order, int n_t
         tg = order.full + q % rest;
         sg = q / rest;
     }
-    tb = tg * 4 + w / 8;
-    sp = sg * 8 + w % 8;
+    tb = tg * order.tbw + w / order.spw;
+    sp = sg * order.spw + w % order.spw;
     return tb < n_token_blocks && sp < n_splits;
 }
 // The next item of the workgroup that holds item v: indices advance by the grid size.  >= n_virtual: none.
