@@ -36,7 +36,11 @@ constexpr int LM_THREADS = 256;
 // Vocabulary tiles per split (at most).  Short splits let a single token block occupy many CUs: at
 // V = 128,256 (501 tiles, 64 splits of 7 or 8) 64 rows take 0.74 ms, against 5.3 ms with 63 tiles per split.
 constexpr int LM_TILES_PER_SPLIT = 8;
-constexpr int LM_BAR = 24;  // group (of 32 per slab) at which the next slab is waited for; 20..28 measure within 2 %
+// Group (of 32 per slab) at which the next slab is waited for.  It lies in the last k-step: the first fragments of
+// the next slab are loaded into the buffer that the k-steps 0 and 2 read, right behind the barrier.  28 measures 2 %
+// slower.
+constexpr int LM_BAR = 24;
+static_assert(LM_BAR >= 24 && LM_BAR <= 28, "the barrier group must lie in the last k-step and leave four groups for the reads");
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr double kLn2 = 0.693147180559945309417232;
 constexpr float kFloor = -1.0e30f;
