@@ -20,16 +20,20 @@ class RolloutExecutor:
         logger.info("Initializing RolloutExecutor on the HIP operators...")
 
     def _select_operators(self) -> Tuple[str, str]:
+        """The two names the reference selects (rollout.py:17-28): the logprob operator and "attention",
+        which is outside the HIP hot path and is answered with the NOT_ON_HIP_PATH name."""
         logp_be = kernel_registry.dispatch("fused_logp")
-        sample_be = kernel_registry.dispatch("sampling")
+        attn_be = kernel_registry.dispatch("attention")
         logger.info_once(f"Selected Logp backend: {logp_be}")
-        logger.info_once(f"Selected Sampling backend: {sample_be}")
-        return logp_be, sample_be
+        logger.info_once(f"Selected Attention backend: {attn_be}")
+        return logp_be, attn_be
 
     def execute_rollout(self):
-        logp_op, sample_op = self._select_operators()
+        """Same result shape as rollout.py:30-35, plus the name of the sampling operator `step` runs."""
+        logp_op, attn_op = self._select_operators()
         logger.info_once(f"Starting rollout via {logp_op}...")
-        return {"status": "success", "kernels": [logp_op, sample_op]}
+        return {"status": "success", "kernels": [logp_op, attn_op],
+                "sampling_kernel": kernel_registry.dispatch("sampling")}
 
     def step(self, logits, uniforms=None):
         """One decode step: sample a token per row of `logits` [B, V] and return (ids, logprobs)."""

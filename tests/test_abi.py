@@ -65,8 +65,10 @@ def test_sampling_argument_checks():
     assert ex(0, None, 0, 128, 128, 1.0, None, 0, None, 1.0, None, None, None, None, None, 0, None) == _hip.KA_OK
     assert ex(7, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 0, None) == _hip.KA_ERR_BAD_ARG   # dtype code
     assert ex(0, p, 2, 128, 128, 0.0, None, 0, None, 1.0, None, p, p, None, None, 0, None) == _hip.KA_ERR_BAD_ARG   # scalar T
-    # a per-row array replaces its scalar, which is then not checked; no GPU here, so the launch itself fails
-    assert ex(0, p, 2, 128, 128, 0.0, p, -1, p, 9.0, p, p, p, None, None, 0, None) == _hip.KA_ERR_HIP
+    # a per-row array replaces its scalar, which is then not checked: the call gets past the scalar checks and
+    # is stopped by the next host check (stride < vocab), so nothing is ever launched on these made-up pointers
+    assert ex(0, p, 2, 128, 64, 0.0, p, -1, p, 9.0, p, p, p, None, None, 0, None) == _hip.KA_ERR_BAD_ARG
+    assert b"stride" in lib.ka_last_error()
 
 
 def test_lmhead_argument_checks_and_workspace_size():

@@ -1,4 +1,6 @@
 """Host side of the op API on a machine without a GPU: construction, validation, pool, side API."""
+import logging
+
 import pytest
 import torch
 
@@ -77,14 +79,48 @@ def test_registry_and_executor():
     assert kernel_registry.dispatch("sampling") == "HIP_SAMPLING"
     assert kernel_registry.dispatch("fused_lm_head_logp") == "HIP_FUSED_LMHEAD_LOGPROB"
     assert kernel_registry.get_op_path(OpBackend.HIP_LOGPROB).endswith("SamplerBackend.compute_logp")
-    with pytest.raises(ValueError):
-        kernel_registry.dispatch("attention")
+    # the reference's dispatch always answers with a name (registry.py:41-55); its callers pass "attention"
+    assert kernel_registry.dispatch("attention") == "NOT_ON_HIP_PATH"
+    assert isinstance(kernel_registry.get_op_path(OpBackend.NOT_ON_HIP_PATH), str)
+    with pytest.raises(ValueError, match="no HIP operator"):
+        kernel_registry.resolve("attention")
     with pytest.raises(ValueError, match="Supported backends"):
         OpBackend["FLASHINFER"]
     fn = kernel_registry.resolve("fused_logp")
     assert fn.__name__ == "compute_logp"
     out = RolloutExecutor({"top_k": 50}).execute_rollout()
-    assert out == {"status": "success", "kernels": ["HIP_LOGPROB", "HIP_SAMPLING"]}
+    assert out["status"] == "success" and out["kernels"] == ["HIP_LOGPROB", "NOT_ON_HIP_PATH"]
+    assert out["sampling_kernel"] == "HIP_SAMPLING"
+
+
+def test_reference_dispatch_smoke_flow():
+    """The flow of the reference's smoke script (rl_engine/tests/test_dispatch.py:9-27), with assertions:
+    once-only logging, the device probe's attributes, dispatch of the two names its callers pass, and the
+    executor's result shape."""
+    from rl_engine.platforms.device import device_ctx
+
+    seen = []
+
+    class Grab(logging.Handler):
+        def emit(self, record):
+            seen.append(record.getMessage())
+
+    h = Grab()
+    logger.addHandler(h)
+    try:
+        logger.info("standard info log")
+        for _ in range(3):
+            logger.info_once("a unique message that appears only once")
+    finally:
+        logger.removeHandler(h)
+    assert seen == ["standard info log", "a unique message that appears only once"]
+    assert isinstance(device_ctx.device_type, str) and isinstance(device_ctx.is_rocm, bool)
+    logp_op = kernel_registry.dispatch("fused_logp")
+    attn_op = kernel_registry.dispatch("attention")
+    assert isinstance(logp_op, str) and isinstance(attn_op, str) and logp_op != attn_op
+    assert OpBackend[logp_op] is OpBackend.HIP_LOGPROB and OpBackend[attn_op] is OpBackend.NOT_ON_HIP_PATH
+    result = RolloutExecutor().execute_rollout()
+    assert result["status"] == "success" and result["kernels"] == [logp_op, attn_op]
 
 
 def test_generate_checks_its_arguments_and_never_falls_back_to_the_cpu():

@@ -145,3 +145,36 @@ def test_lmhead_backward_oracle_forms_agree_and_match_finite_differences():
         e = torch.zeros_like(w0); e[r, c] = eps
         fd = (loss(h0, w0 + e) - loss(h0, w0 - e)) / (2 * eps)
         assert abs(fd.item() - dw_c[r, c].item()) < 1e-7
+
+
+def test_lmhead_oracle_is_the_logprob_oracle_on_the_linear_layer():
+    """lmhead_logprob_ref is pinned two ways: against logprob_f64 on an fp64 F.linear, and against a
+    pure-Python evaluation (explicit dot products + math.fsum) that shares no code with it, so that a
+    transposed weight, a wrong gather index or a dropped maximum would fail."""
+    g = torch.Generator().manual_seed(21)
+    hidden = torch.randn(37, 64, generator=g).bfloat16()
+    weight = (torch.randn(301, 64, generator=g) * 0.2).bfloat16()
+    ids = torch.randint(0, 301, (37,), generator=g)
+    logits64 = torch.nn.functional.linear(hidden.double(), weight.double())
+    want64 = O.logprob_f64(logits64, ids)
+    got64 = O.lmhead_logprob_ref(hidden, weight, ids, dtype=torch.float64, chunk_rows=16)   # ragged last chunk
+    assert got64.shape == (37,) and got64.dtype == torch.float64
+    assert (got64 - want64).abs().max().item() < 1e-12
+    got32 = O.lmhead_logprob_ref(hidden, weight, ids)
+    assert got32.dtype == torch.float32 and (got32.double() - want64).abs().max().item() < 2e-5
+    # leading dimensions are kept
+    assert torch.equal(O.lmhead_logprob_ref(hidden[:36].view(4, 9, 64), weight, ids[:36].view(4, 9), torch.float64),
+                       got64[:36].view(4, 9))
+
+    # non-square [3,8] x [5,8] case, rows and targets all different, evaluated in plain Python
+    h = (torch.randn(3, 8, generator=g) * 2).bfloat16()
+    w = torch.randn(5, 8, generator=g).bfloat16()
+    t = torch.tensor([4, 0, 2])
+    got = O.lmhead_logprob_ref(h, w, t, dtype=torch.float64)
+    hl, wl = h.double().tolist(), w.double().tolist()
+    for r in range(3):
+        row = [math.fsum(hl[r][k] * wl[v][k] for k in range(8)) for v in range(5)]
+        assert abs(got[r].item() - O.logprob_bruteforce(row, int(t[r]))) < 1e-12
+    # closed form: zero hidden row -> uniform distribution over the vocabulary
+    z = O.lmhead_logprob_ref(torch.zeros(1, 8, dtype=torch.bfloat16), w, torch.tensor([3]), torch.float64)
+    assert abs(z.item() + math.log(5)) < 1e-14

@@ -90,7 +90,7 @@ def brute_force_row(y, k, p, u):
     for i in sorted(kept):
         cum += w[i]
         if Fraction(cum) > Fraction(f32(u)) * zb:
-            return i, len(order), len(kept)
+            return i, len(order), len(kept), w[i], zb
     raise AssertionError("no index selected")
 
 
@@ -113,9 +113,47 @@ def test_exact_oracle_matches_pure_python_definition(dtype, k, p, temp):
     got, info = exact.sample(logits, temp, k, p, u, return_info=True)
     y = exact.scale(logits, temp)
     for r in range(logits.shape[0]):
-        want, na, nb = brute_force_row(y[r].tolist(), k, p, float(u[r]))
+        want, na, nb, w_pick, zb = brute_force_row(y[r].tolist(), k, p, float(u[r]))
         assert got[r].item() == want, (r, info[r])
         assert (info[r]["n_topk"], info[r]["n_kept"]) == (na, nb)
+        assert (info[r]["w_pick"], info[r]["z_kept"]) == (w_pick, zb)
+
+
+def test_drawn_token_logprob_matches_pure_python_definition():
+    """sample_rows' log-probability (log of w_pick / z_kept) against the brute-force masses, with per-row
+    parameters, a cut that falls inside a tie group, and closed forms."""
+    logits, u = coarse_rows(12, 61, seed=99, dtype=torch.bfloat16)
+    # row 0: five entries tie at the maximum and top_p cuts inside the group: mass before the third is
+    # 2/5 > 0.35, so exactly two survive and either has probability 1/2
+    logits[0, :] = -3.0
+    logits[0, [4, 9, 20, 33, 50]] = 2.0
+    temps = [1.0, 0.7, 1.3, 1.0, 0.5, 2.0, 1.0, 0.7, 1.0, 1.0, 0.9, 1.0]
+    ks = [0, 5, 5, 0, 17, 3, 1, 200, 0, 61, 7, 2]
+    ps = [0.35, 0.9, 1.0, 0.8, 0.05, 1.0, 0.5, 0.95, 1.0, 0.6, 0.3, 0.99]
+    ids, lps = exact.sample_rows(logits, temps, ks, ps, u)
+    for r in range(12):
+        y = exact.scale(logits[r:r + 1], temps[r])[0].tolist()
+        want, _, nb, w_pick, zb = brute_force_row(y, ks[r], ps[r], float(u[r]))
+        assert ids[r].item() == want
+        true = math.log(Fraction(w_pick, zb))
+        assert abs(lps[r].item() - true) < 1e-12, (r, lps[r].item(), true)
+        assert lps[r].item() <= 0.0
+        if nb == 1:
+            assert lps[r].item() == 0.0
+    _, info = exact.sample(logits[:1], 1.0, 0, 0.35, u[:1], return_info=True)
+    assert info[0]["n_kept"] == 2 and ids[0].item() in (4, 9)
+    assert abs(lps[0].item() + math.log(2)) < 1e-12
+    # closed forms: uniform survivors -> -log(count); top_k = 1 -> 0
+    flat = torch.zeros(3, 10, dtype=torch.float32)
+    _, lp = exact.sample_rows(flat, None, [0, 0, 1], [1.0, 0.3, 1.0], torch.tensor([0.1, 0.6, 0.9]))
+    assert abs(lp[0].item() + math.log(10)) < 1e-12 and abs(lp[1].item() + math.log(4)) < 1e-12
+    assert abs(lp[2].item() + math.log(10)) < 1e-12          # ten-way tie at the maximum: top_k = 1 keeps all
+    # the probabilities of all survivors sum to one (stratified uniforms visit every survivor)
+    row = (torch.randn(1, 40, generator=torch.Generator().manual_seed(8)) * 2).float()
+    n = 2000
+    got_ids, got_lp = exact.sample_rows(row.expand(n, 40).contiguous(), 0.8, 9, 0.9, (torch.arange(n) + 0.5) / n)
+    per_id = {int(i): float(l) for i, l in zip(got_ids, got_lp)}
+    assert abs(sum(math.exp(v) for v in per_id.values()) - 1.0) < 1e-9
 
 
 # ---------------------------------------------------------------- closed forms
