@@ -71,13 +71,18 @@ int ka_logprob_f32(const void *logits, int64_t n_rows, int64_t vocab, int64_t ro
  */
 int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
                             const int64_t *ids, float *out, float *entropy, void *hip_stream);
+int ka_logprob_entropy_f16(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                           const int64_t *ids, float *out, float *entropy, void *hip_stream);
+int ka_logprob_entropy_f32(const void *logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                           const int64_t *ids, float *out, float *entropy, void *hip_stream);
 
 /*
  * Backward of ka_logprob_*:
  *     dlogits[r, v] = grad[r] * ((v == ids[r]) - softmax(logits[r, :])[v])
  * in the logits' dtype.  logp is the forward result for the same (logits, ids);
  * the row's log-sum-exp is recovered from it, so each logit is read once and
- * its gradient written once.  dlogits may be the logits buffer itself (same
+ * its gradient written once (a row whose target logit is -inf, where logp is
+ * -inf too, is read twice: its log-sum-exp is recomputed).  dlogits may be the logits buffer itself (same
  * stride): the gradient then overwrites the logits and no second tensor of
  * their size exists.  No counterpart in the reference, whose operators run under
  * torch.inference_mode() (rl_engine/kernels/sampling.py:38,91); this is the

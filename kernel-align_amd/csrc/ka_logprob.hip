@@ -207,6 +207,18 @@ KA_EXPORT int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_
     return ka::launch<ka::Bf16, true>(logits, n_rows, vocab, row_stride, ids, out, entropy, hip_stream);
 }
 
+KA_EXPORT int ka_logprob_entropy_f16(const void *logits, int64_t n_rows, int64_t vocab,
+                                     int64_t row_stride, const int64_t *ids, float *out,
+                                     float *entropy, void *hip_stream) {
+    return ka::launch<ka::F16, true>(logits, n_rows, vocab, row_stride, ids, out, entropy, hip_stream);
+}
+
+KA_EXPORT int ka_logprob_entropy_f32(const void *logits, int64_t n_rows, int64_t vocab,
+                                     int64_t row_stride, const int64_t *ids, float *out,
+                                     float *entropy, void *hip_stream) {
+    return ka::launch<ka::F32, true>(logits, n_rows, vocab, row_stride, ids, out, entropy, hip_stream);
+}
+
 // ---------------------------------------------------------------------------
 // Backward of the per-token logprob:
 //     dlogits[r, v] = grad[r] * ((v == ids[r]) - softmax(logits[r, :])[v])
@@ -215,6 +227,9 @@ KA_EXPORT int ka_logprob_entropy_bf16(const void *logits, int64_t n_rows, int64_
 // gradient written once, in the logits' dtype.  dlogits may alias logits (each
 // element is read and then written by the same lane), so the gradient of a
 // [G, L, V] tensor needs no second tensor of that size.
+// A target whose logit is -inf (a masked entry) has logp = -inf, from which the
+// log-sum-exp cannot be recovered: such a row takes one more pass that
+// recomputes it, and gets the finite gradient -g * softmax autograd gives.
 // ---------------------------------------------------------------------------
 namespace ka {
 namespace {
@@ -269,7 +284,11 @@ __global__ __launch_bounds__(THREADS) void logprob_backward_rows(const typename 
                                                                  const float *__restrict__ grad,
                                                                  typename T::raw_t *dlogits, int64_t d_stride) {
     constexpr int EPV = T::kPerVec;
+    constexpr int NWAVES = THREADS / kWave;
     __shared__ float s_lse;
+    __shared__ int s_masked;
+    __shared__ float red_a[NWAVES];
+    __shared__ float red_b[NWAVES];
     const int tid = threadIdx.x;
     for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
         const typename T::raw_t *rp = logits + row * row_stride;
@@ -279,8 +298,36 @@ __global__ __launch_bounds__(THREADS) void logprob_backward_rows(const typename 
         const float g = grad[row];
         // lse = x_t - logp; an id outside the vocabulary has no defined forward value: its row gets NaN.
         // One lane reads x_t and the barrier comes before any store, because dlogits may be the logits.
-        if (tid == 0) s_lse = id_ok ? T::widen(rp[id]) - logp[row] : __builtin_nanf("");
+        if (tid == 0) {
+            const float x_t = id_ok ? T::widen(rp[id]) : __builtin_nanf("");
+            s_lse = x_t - logp[row];
+            s_masked = id_ok && x_t == -__builtin_inff();
+        }
         __syncthreads();
+        if (s_masked) {  // workgroup-uniform and rare: recompute the row's log-sum-exp (before any store)
+            RowState st{kFloor, kFloor * kLog2e, 0.0f, 0.0f};
+            for (int i = tid; i < vocab; i += THREADS) {
+                const float xs[1] = {T::widen(rp[i])};
+                fold<1, false>(st, xs);
+            }
+            const float wm = wave_max(st.ml2);
+            if ((tid & (kWave - 1)) == 0) red_a[tid / kWave] = wm;
+            __syncthreads();
+            float big = red_a[0];
+#pragma unroll
+            for (int w = 1; w < NWAVES; ++w) big = fmaxf(big, red_a[w]);
+            const float ws = wave_sum(st.s * fast_exp2(st.ml2 - big));
+            if ((tid & (kWave - 1)) == 0) red_b[tid / kWave] = ws;
+            __syncthreads();
+            if (tid == 0) {
+                float total = red_b[0];
+#pragma unroll
+                for (int w = 1; w < NWAVES; ++w) total += red_b[w];
+                // a row of nothing but -inf keeps NaN, as softmax of such a row does
+                s_lse = total > 0.0f ? float((double(big) + log2(double(total))) * kLn2) : __builtin_nanf("");
+            }
+            __syncthreads();
+        }
         const float lse = s_lse;
         const float nl2 = -lse * kLog2e;
         const float ng = -g;

@@ -20,6 +20,7 @@ LIB_NAME = "libkernel_align_hip.so"
 ENV_LIB = "KERNEL_ALIGN_HIP_LIB"
 
 _LOGPROB_ARGS = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
+_ENTROPY_ARGS = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
 _BACKWARD_ARGS = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]
 _SAMPLE_ARGS = [c_void_p, c_int64, c_int64, c_int64, c_float, c_int32, c_float, c_void_p, c_void_p,
                 c_void_p, c_size_t, c_void_p]
@@ -32,8 +33,9 @@ SIGNATURES = {
     "ka_logprob_bf16": (c_int, _LOGPROB_ARGS),
     "ka_logprob_f16": (c_int, _LOGPROB_ARGS),
     "ka_logprob_f32": (c_int, _LOGPROB_ARGS),
-    "ka_logprob_entropy_bf16": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
-                                        c_void_p]),
+    "ka_logprob_entropy_bf16": (c_int, _ENTROPY_ARGS),
+    "ka_logprob_entropy_f16": (c_int, _ENTROPY_ARGS),
+    "ka_logprob_entropy_f32": (c_int, _ENTROPY_ARGS),
     "ka_logprob_backward_bf16": (c_int, _BACKWARD_ARGS),
     "ka_logprob_backward_f16": (c_int, _BACKWARD_ARGS),
     "ka_logprob_backward_f32": (c_int, _BACKWARD_ARGS),

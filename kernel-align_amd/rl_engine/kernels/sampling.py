@@ -23,6 +23,8 @@ DEFAULT_CHUNK_TOKENS = 8192
 
 _LOGPROB_FN = {torch.bfloat16: "ka_logprob_bf16", torch.float16: "ka_logprob_f16",
                torch.float32: "ka_logprob_f32"}
+_ENTROPY_FN = {torch.bfloat16: "ka_logprob_entropy_bf16", torch.float16: "ka_logprob_entropy_f16",
+               torch.float32: "ka_logprob_entropy_f32"}
 _BACKWARD_FN = {torch.bfloat16: "ka_logprob_backward_bf16", torch.float16: "ka_logprob_backward_f16",
                 torch.float32: "ka_logprob_backward_f32"}
 _DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
@@ -33,6 +35,14 @@ _SAMPLE_FN = {torch.bfloat16: "ka_sample_topk_topp_bf16", torch.float16: "ka_sam
 def _require_gpu(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(f"{name} must live on the GPU: rl_engine has no CPU path (got {t.device})")
+
+
+def _chunk_rows(chunk_tokens) -> int:
+    """Rows per launch of a chunked operator; anything below one row would make the launch loop empty."""
+    chunk = DEFAULT_CHUNK_TOKENS if chunk_tokens is None else int(chunk_tokens)
+    if chunk < 1:
+        raise ValueError(f"chunk_tokens must be >= 1 (got {chunk_tokens})")
+    return chunk
 
 
 def _rows_view(logits: torch.Tensor) -> torch.Tensor:
@@ -89,9 +99,7 @@ class SamplerBackend(nn.Module):
         n_rows, vocab = rows.shape
         ids = token_ids.to(device=logits.device, dtype=torch.int64).contiguous().view(-1)
         out = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
-        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
-        if chunk < 1:
-            raise ValueError("chunk_tokens must be >= 1")
+        chunk = _chunk_rows(chunk_tokens)
         row_stride = rows.stride(0) if n_rows > 1 else vocab
         esize = rows.element_size()
         with torch.cuda.device(logits.device):
@@ -108,27 +116,31 @@ class SamplerBackend(nn.Module):
 
     @torch.inference_mode()
     def compute_logp_entropy(self, logits, token_ids, chunk_tokens=None):
-        """compute_logp plus the entropy of every row's softmax, from the same single pass (bf16)."""
+        """compute_logp plus the entropy of every row's softmax, from the same single pass (bf16 / fp16 / fp32)."""
         _require_gpu(logits, "logits")
-        if logits.dtype != torch.bfloat16:
-            raise TypeError("compute_logp_entropy takes bf16 logits")
+        fn_name = _ENTROPY_FN.get(logits.dtype)
+        if fn_name is None:
+            raise TypeError(f"unsupported logits dtype {logits.dtype}")
+        if logits.dim() < 2:
+            raise ValueError("logits must be [..., V]")
         if tuple(token_ids.shape) != tuple(logits.shape[:-1]):
             raise ValueError("token_ids shape must equal logits.shape[:-1]")
+        chunk = _chunk_rows(chunk_tokens)
+        fn = getattr(self._lib, fn_name)
         rows = _rows_view(logits)
         n_rows, vocab = rows.shape
         ids = token_ids.to(device=logits.device, dtype=torch.int64).contiguous().view(-1)
         out = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
         ent = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
-        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
         row_stride = rows.stride(0) if n_rows > 1 else vocab
+        esize = rows.element_size()
         with torch.cuda.device(logits.device):
             stream = torch.cuda.current_stream().cuda_stream
             for start in range(0, n_rows, chunk):
                 n = min(chunk, n_rows - start)
-                status = self._lib.ka_logprob_entropy_bf16(
-                    rows.data_ptr() + start * row_stride * 2, n, vocab, row_stride,
-                    ids.data_ptr() + start * 8, out.data_ptr() + start * 4, ent.data_ptr() + start * 4, stream)
-                _hip.check(status, "ka_logprob_entropy_bf16")
+                status = fn(rows.data_ptr() + start * row_stride * esize, n, vocab, row_stride,
+                            ids.data_ptr() + start * 8, out.data_ptr() + start * 4, ent.data_ptr() + start * 4, stream)
+                _hip.check(status, fn_name)
         shape = tuple(logits.shape[:-1])
         return out.view(shape), ent.view(shape)
 
@@ -162,7 +174,7 @@ class SamplerBackend(nn.Module):
         row_stride = rows.stride(0) if n_rows > 1 else vocab
         out_stride = out_rows.stride(0) if n_rows > 1 else vocab
         esize = rows.element_size()
-        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
+        chunk = _chunk_rows(chunk_tokens)
         fn = getattr(self._lib, fn_name)
         with torch.cuda.device(logits.device):
             stream = torch.cuda.current_stream().cuda_stream
@@ -379,9 +391,7 @@ class SamplerBackend(nn.Module):
         n_rows = h2.shape[0]
         ids = token_ids.to(device=hidden.device, dtype=torch.int64).contiguous().view(-1)
         g = grad_logp.to(device=hidden.device, dtype=torch.float32).contiguous().view(-1)
-        chunk = int(chunk_tokens or DEFAULT_CHUNK_TOKENS)
-        if chunk < 1:
-            raise ValueError("chunk_tokens must be >= 1")
+        chunk = _chunk_rows(chunk_tokens)
         if dweight_dtype not in (torch.float32, torch.bfloat16):
             raise TypeError("dweight_dtype must be torch.float32 or torch.bfloat16")
         dhidden = torch.empty_like(h2)

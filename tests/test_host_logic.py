@@ -131,3 +131,14 @@ def test_generate_checks_its_arguments_and_never_falls_back_to_the_cpu():
         executor.generate(lambda ids: None, torch.zeros(2, 3, dtype=torch.int64), 2, uniforms=torch.zeros(2, 3))
     with pytest.raises((RuntimeError, ValueError)):     # CPU logits are refused by the operators
         executor.generate(lambda ids: torch.zeros(2, 16), torch.zeros(2, 3, dtype=torch.int64), 1)
+
+
+def test_chunk_rows_validation():
+    """Every chunked operator takes its launch granularity from one checked helper: a value below one row would
+    make the launch loop empty and return uninitialised memory."""
+    from rl_engine.kernels.sampling import DEFAULT_CHUNK_TOKENS, _chunk_rows
+
+    assert _chunk_rows(None) == DEFAULT_CHUNK_TOKENS and _chunk_rows(7) == 7
+    for bad in (0, -1, -8192):
+        with pytest.raises(ValueError, match="chunk_tokens"):
+            _chunk_rows(bad)

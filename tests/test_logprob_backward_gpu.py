@@ -66,3 +66,25 @@ def test_unaligned_rows_and_determinism(sampler):
                        for s in range(0, 16, 4)])
     whole = sampler.compute_logp_backward(big[:, :4096], ids, sampler.compute_logp(big[:, :4096], ids), grad)
     assert torch.equal(parts, whole)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_masked_target_gets_the_finite_gradient_autograd_gives(sampler, dtype):
+    """A target whose logit is -inf has logp = -inf, so the log-sum-exp cannot be recovered from it: the kernel
+    recomputes it for such a row and returns -g * softmax (what autograd gives), not NaN."""
+    logits, ids, grad = make(12, 5003, dtype, 77)
+    logits[3, ids[3]] = float("-inf")
+    logits[8, 100:] = float("-inf")
+    ids[8] = 4000                                  # masked target in a row with a masked tail
+    dl, di, dg = logits.cuda(), ids.cuda(), grad.cuda()
+    logp = sampler.compute_logp(dl, di)
+    assert logp[3].item() == float("-inf") and logp[8].item() == float("-inf")
+    got = sampler.compute_logp_backward(dl, di, logp, dg).cpu()
+    assert torch.isfinite(got).all()
+    check(got, logits, ids, grad)
+    auto = O.logprob_backward_ref(logits, ids, grad, dtype=torch.float64)
+    assert torch.isfinite(auto).all() and (got.double() - auto).abs().max().item() < 2e-2
+    inplace = sampler.compute_logp_backward(dl.clone(), di, logp, dg, inplace=True)
+    assert torch.equal(inplace.cpu(), got)
+    with pytest.raises(ValueError, match="chunk_tokens"):
+        sampler.compute_logp_backward(dl, di, logp, dg, chunk_tokens=-1)

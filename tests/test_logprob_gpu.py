@@ -144,6 +144,24 @@ def test_entropy_variant(sampler):
     assert (ent2.cpu().double() - O.entropy_f64(masked)).abs().max().item() <= TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_entropy_variant_other_dtypes(sampler, dtype):
+    """fp16 and fp32 logits through the same pass (aligned rows, and an unaligned view that takes the scalar loads)."""
+    g = torch.Generator().manual_seed(17)
+    logits = (torch.randn(96, 40003, generator=g) * 3).to(dtype)
+    logits[::7, 11] = 20.0
+    logits[5, 2000:] = -math.inf
+    ids = torch.randint(0, 2000, (96,), generator=g)
+    aligned = logits[:, :40000].contiguous()
+    for x in (aligned, logits[:, 3:40003]):
+        lp, ent = sampler.compute_logp_entropy(x.cuda(), ids.cuda())
+        assert torch.equal(lp, sampler.compute_logp(x.cuda(), ids.cuda()))
+        assert (lp.cpu().double() - O.logprob_f64(x, ids)).abs().max().item() <= 2e-5
+        assert (ent.cpu().double() - O.entropy_f64(x)).abs().max().item() <= TOL
+    with pytest.raises(ValueError, match="chunk_tokens"):
+        sampler.compute_logp_entropy(aligned.cuda(), ids.cuda(), chunk_tokens=-4)
+
+
 def test_full_size_grpo_group(sampler):
     """[256, 512, 128256] bf16 (33.6 GB): parity on sampled blocks, invariance on everything."""
     n_rows, vocab, blk = 256 * 512, 128256, 2048
