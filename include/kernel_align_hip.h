@@ -187,6 +187,22 @@ int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t
                            int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
                            size_t workspace_bytes, void *hip_stream);
 
+/*
+ * ka_lmhead_logprob_bf16 for callers that cannot allocate device memory or bring a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same kernels, same results bit
+ * for bit; the per-split partials go to a static array in device memory (KA_LMHEAD_STATIC_SCRATCH_BYTES,
+ * one copy on every GPU the library runs on, held until the process ends) instead of a workspace, and the
+ * call makes no hipMalloc / hipFree.  It has no counterpart in the reference.
+ * Limit: ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab) <= KA_LMHEAD_STATIC_SCRATCH_BYTES (16,384
+ * rows at a vocabulary of 128,256); more returns KA_ERR_WORKSPACE and nothing is launched.  Every call on
+ * a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on
+ * one stream are ordered and safe.  The first call on a device looks the array's address up (one
+ * hipGetSymbolAddress and the kernels' attribute set-up), so make one call per device before capturing.
+ */
+#define KA_LMHEAD_STATIC_SCRATCH_BYTES (16u << 20)
+int ka_lmhead_logprob_bf16_noalloc(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                   int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

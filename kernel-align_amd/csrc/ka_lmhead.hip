@@ -20,6 +20,8 @@
 //     rows); every (token block, split) writes one (max, sum, target logit)
 //     partial per token and a second kernel folds the partials in split order.
 // Logits stay in fp32 (the accumulators are not rounded to bf16).
+#include <mutex>
+
 #include "ka_common.h"
 
 namespace ka {
@@ -487,12 +489,63 @@ KA_EXPORT size_t ka_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, i
     return size_t(ka::splits_for(vocab)) * size_t(n_rows) * sizeof(ka::Partial);
 }
 
-KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
-                                     int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
-                                     size_t workspace_bytes, void *hip_stream) {
-    using namespace ka;
-    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead: n_rows %lld < 0", (long long)n_rows);
-    if (n_rows == 0) return KA_OK;
+namespace ka {
+namespace {
+
+// Scratch of ka_lmhead_logprob_bf16_noalloc: the partials of one call live here instead of in a caller's workspace.
+// Every GPU the library runs on holds its own copy of the array until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress: kernels are given the device address looked up below.
+constexpr size_t LM_STATIC_SCRATCH_BYTES = KA_LMHEAD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char lm_static_scratch[LM_STATIC_SCRATCH_BYTES];
+
+// What the launch needs to know about a device, looked up once per device with that device current.
+struct LmDevice {
+    bool ready = false;          // cus is valid and both kernels have their LDS size reserved on this device
+    bool scratch_ready = false;  // scratch is valid
+    int cus = 0;
+    void *scratch = nullptr;     // device address of this device's lm_static_scratch
+};
+constexpr int LM_MAX_DEVICES = 64;
+LmDevice g_lm_device[LM_MAX_DEVICES];
+std::mutex g_lm_device_mutex;
+
+// Fills `out` with the current device's record (a copy: the table is only touched under the mutex).
+int lm_current_device(bool need_scratch, LmDevice &out) {
+    int device = 0;
+    hipError_t rc = hipGetDevice(&device);
+    if (rc != hipSuccess) return check_hip(rc, "lmhead: hipGetDevice");
+    if (device < 0 || device >= LM_MAX_DEVICES) return fail(KA_ERR_UNSUPPORTED, "lmhead: device index %d", device);
+    std::lock_guard<std::mutex> lock(g_lm_device_mutex);
+    LmDevice &d = g_lm_device[device];
+    if (!d.ready) {
+        int cus = 0;
+        rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+        if (rc != hipSuccess) return check_hip(rc, "lmhead: querying the CU count");
+        // the attribute belongs to the device, so it is set once per device and not once per process
+        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials<false>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
+        if (rc == hipSuccess)
+            rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials<true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
+        if (rc != hipSuccess) return check_hip(rc, "lmhead: reserving 131 KB of LDS");
+        d.cus = cus;
+        d.ready = true;
+    }
+    if (need_scratch && !d.scratch_ready) {
+        void *ptr = nullptr;
+        rc = hipGetSymbolAddress(&ptr, HIP_SYMBOL(lm_static_scratch));
+        if (rc != hipSuccess || ptr == nullptr)
+            return check_hip(rc != hipSuccess ? rc : hipErrorInvalidSymbol, "lmhead: address of the static scratch array");
+        d.scratch = ptr;
+        d.scratch_ready = true;
+    }
+    out = d;
+    return KA_OK;
+}
+
+// Argument checks shared by the two entry points (everything except the workspace).
+int lm_check_args(const void *hidden, const void *weight, const int64_t *ids, const float *out, int64_t n_rows,
+                  int64_t hidden_dim, int64_t vocab) {
     if (hidden == nullptr || weight == nullptr || ids == nullptr || out == nullptr)
         return fail(KA_ERR_BAD_ARG, "lmhead: null hidden / weight / ids / out pointer");
     if (hidden_dim < 8 || vocab < 1) return fail(KA_ERR_BAD_ARG, "lmhead: hidden_dim %lld, vocab %lld", (long long)hidden_dim, (long long)vocab);
@@ -502,9 +555,12 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
         return fail(KA_ERR_UNSUPPORTED, "lmhead: hidden and weight must be 16-byte aligned");
     if (n_rows >= (int64_t(1) << 31) || vocab >= (int64_t(1) << 31) || hidden_dim >= (int64_t(1) << 31))
         return fail(KA_ERR_UNSUPPORTED, "lmhead: a dimension does not fit 31 bits");
-    const size_t need = ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab);
-    if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
-        return fail(KA_ERR_WORKSPACE, "lmhead: workspace of %zu B (16-byte aligned) needed, got %zu B", need, workspace_bytes);
+    return KA_OK;
+}
+
+// Enqueues the two kernels; `partials` holds ka_lmhead_workspace_bytes(n_rows, ., vocab) bytes of device memory.
+int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const int64_t *ids, float *out,
+              int64_t n_rows, int64_t hidden_dim, int64_t vocab, Partial *partials, hipStream_t stream) {
     const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
     const int n_splits = splits_for(vocab);
     const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
@@ -512,20 +568,9 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     if (n_virtual >= (int64_t(1) << 30)) return fail(KA_ERR_UNSUPPORTED, "lmhead: too many work items");
     // One workgroup per CU (a workgroup takes a CU's LDS and registers); each walks its items.  256 workgroups
     // keep item v on XCD v % 8 and at one position of its super-tiles.
-    int device = 0, cus = 0;
-    hipError_t dev_rc = hipGetDevice(&device);
-    if (dev_rc == hipSuccess) dev_rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
-    if (dev_rc != hipSuccess) return check_hip(dev_rc, "lmhead: querying the CU count");
-    const int64_t resident = cus >= 256 ? 256 : (cus >= 8 ? cus / 8 * 8 : 8);
+    const int64_t resident = dev.cus >= 256 ? 256 : (dev.cus >= 8 ? dev.cus / 8 * 8 : 8);
     const int64_t grid = n_virtual < resident ? n_virtual : resident;
-    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    Partial *partials = static_cast<Partial *>(workspace);
     const bool wide = n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32);
-    const void *kernel = wide ? reinterpret_cast<const void *>(lmhead_partials<true>)
-                              : reinterpret_cast<const void *>(lmhead_partials<false>);
-    // set on every call rather than once per process: the attribute belongs to the current device
-    const hipError_t attr_rc = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
-    if (attr_rc != hipSuccess) return check_hip(attr_rc, "lmhead: reserving 131 KB of LDS");
     if (wide)
         hipLaunchKernelGGL(lmhead_partials<true>, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                            static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
@@ -539,4 +584,46 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids, out,
                        int(n_rows), int(vocab), n_splits);
     return check_hip(hipGetLastError(), "lmhead combine launch");
+}
+
+}  // namespace
+}  // namespace ka
+
+KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                     int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
+                                     size_t workspace_bytes, void *hip_stream) {
+    using namespace ka;
+    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead: n_rows %lld < 0", (long long)n_rows);
+    if (n_rows == 0) return KA_OK;
+    int rc = lm_check_args(hidden, weight, ids, out, n_rows, hidden_dim, vocab);
+    if (rc != KA_OK) return rc;
+    const size_t need = ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab);
+    if (workspace == nullptr || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return fail(KA_ERR_WORKSPACE, "lmhead: workspace of %zu B (16-byte aligned) needed, got %zu B", need, workspace_bytes);
+    LmDevice dev;
+    rc = lm_current_device(false, dev);
+    if (rc != KA_OK) return rc;
+    return lm_launch(dev, hidden, weight, ids, out, n_rows, hidden_dim, vocab, static_cast<Partial *>(workspace),
+                     static_cast<hipStream_t>(hip_stream));
+}
+
+KA_EXPORT int ka_lmhead_logprob_bf16_noalloc(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                             int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *hip_stream) {
+    using namespace ka;
+    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead: n_rows %lld < 0", (long long)n_rows);
+    if (n_rows == 0) return KA_OK;
+    int rc = lm_check_args(hidden, weight, ids, out, n_rows, hidden_dim, vocab);
+    if (rc != KA_OK) return rc;
+    const size_t need = ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab);
+    if (need > LM_STATIC_SCRATCH_BYTES)
+        return fail(KA_ERR_WORKSPACE,
+                    "lmhead (noalloc): %lld rows x vocab %lld need %zu B of partials, the static scratch holds %zu B; "
+                    "pass fewer rows per call or use ka_lmhead_logprob_bf16 with a workspace",
+                    (long long)n_rows, (long long)vocab, need, LM_STATIC_SCRATCH_BYTES);
+    LmDevice dev;
+    rc = lm_current_device(true, dev);
+    if (rc != KA_OK) return rc;
+    // Nothing in the scratch has to start at zero: every partial the fold reads is written by this call's first kernel.
+    return lm_launch(dev, hidden, weight, ids, out, n_rows, hidden_dim, vocab, static_cast<Partial *>(dev.scratch),
+                     static_cast<hipStream_t>(hip_stream));
 }

@@ -91,6 +91,16 @@ def test_lmhead_argument_checks_and_workspace_size():
     assert call(p, p, p, p, 4, 4096, 128256, None, 0, None) == _hip.KA_ERR_WORKSPACE
     assert call(p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
     assert b"workspace" in lib.ka_last_error()
+    # the variant without a workspace argument: same checks, and a size limit instead of a workspace check
+    na = lib.ka_lmhead_logprob_bf16_noalloc
+    assert na(None, None, None, None, 0, 4096, 128256, None) == _hip.KA_OK
+    assert na(None, p, p, p, 4, 4096, 128256, None) == _hip.KA_ERR_BAD_ARG
+    assert na(p, p, p, p, 4, 100, 128256, None) == _hip.KA_ERR_UNSUPPORTED
+    assert ws(16384, 4096, 128256) == _hip.LMHEAD_STATIC_SCRATCH_BYTES
+    assert na(p, p, p, p, 16385, 4096, 128256, None) == _hip.KA_ERR_WORKSPACE
+    assert b"static scratch" in lib.ka_last_error()
+    header = HEADER.read_text()
+    assert "#define KA_LMHEAD_STATIC_SCRATCH_BYTES (16u << 20)" in header
 
 
 def test_grpo_and_backward_argument_checks():
