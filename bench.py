@@ -26,18 +26,33 @@ for _p in (REPO, REPO / "kernel-align_amd"):
 HBM_PEAK_GBPS = 8000.0
 G, L, V = 256, 512, 128256
 BYTES_PER_TOKEN = 2 * V + 8 + 4
-# HBM traffic of the logprob kernel per token, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this
-# program (profiles/logprob_rows_bf16_G256_L512_V128256.txt): 2 x 1,026,607.7 KiB fetched + 258.3 KiB
-# written per 8192-row launch.
-MEASURED_TRAFFIC_PER_TOKEN = (2 * 1026607.7 + 258.3) * 1024 / 8192
+# HBM traffic per launch of each kernel, in bytes.  These are NOT measured by this program: they come from
+# separate rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (one counter per run), scaled by
+# what the counters read for a plain 1 GiB copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000), and
+# are repeated here with their source so that a reader can tell them from live figures.  A kernel whose code
+# changed after its profile was taken reports null until the profile is redone.
+STATIC_TRAFFIC = {
+    "logprob_rows": ((2 * 1026607.7 + 258.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt"),
+    "logprob_backward_rows": ((2 * 1027116 + 2052133) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt"),
+    "sample_rows": (None, "profiles/sample_rows_bf16_B64-256_V128256.txt"),
+    "lmhead_partials": (None, "profiles/lmhead_partials_bf16_N32768_H4096_V128256.txt"),
+}
+PARITY_TOL = 1e-4
+
+
+def traffic_fields(kernel: str) -> dict:
+    value, source = STATIC_TRAFFIC[kernel]
+    return {"traffic": value, "traffic_source": f"static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in {source}"
+            if value is not None else "not collected for the current build of this kernel"}
 
 
 def log(msg: str) -> None:
     print(msg, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(logits, ids, sample_rows: int):
-    """Time the fp32 torch CPU oracle on `sample_rows` rows taken evenly from the tensor."""
+def cpu_baseline(logits, ids, gpu_out, sample_rows: int):
+    """Time the fp32 torch CPU oracle on `sample_rows` rows taken evenly from the tensor, and compare what it
+    returns with the GPU result of the timed run on those rows (all of them by default)."""
     import torch
     from oracle import logprob_ref
 
@@ -45,13 +60,23 @@ def cpu_baseline(logits, ids, sample_rows: int):
     n_blocks = max(1, sample_rows // blk)
     total_rows = logits.shape[0]
     starts = [int(i * (total_rows - blk) / max(1, n_blocks - 1)) // blk * blk for i in range(n_blocks)]
-    elapsed, rows, max_err = 0.0, 0, None
+    elapsed, rows, max_err, spike_err, spike_rows, spike_hits = 0.0, 0, 0.0, 0.0, 0, 0
+    flat_out = gpu_out.reshape(-1)
     for s in starts:
         lc, ic = logits[s:s + blk].cpu(), ids[s:s + blk].cpu()
         t0 = time.perf_counter()
-        logprob_ref.logprob_ref(lc, ic)
+        want = logprob_ref.logprob_ref(lc, ic)
         elapsed += time.perf_counter() - t0
         rows += lc.shape[0]
+        err = (flat_out[s:s + blk].cpu() - want).abs()
+        max_err = max(max_err, err.max().item())
+        # rows that carry a +25 spike (N(0, 3^2) stays below 16 over 128,256 draws)
+        spike_col = lc.argmax(dim=-1)
+        is_spike = lc.gather(-1, spike_col.unsqueeze(-1)).squeeze(-1).float() >= 24.0
+        if bool(is_spike.any()):
+            spike_rows += int(is_spike.sum())
+            spike_hits += int((is_spike & (spike_col == ic)).sum())
+            spike_err = max(spike_err, err[is_spike].max().item())
     return {
         "value": rows / elapsed,
         "unit": "tokens/s",
@@ -59,6 +84,9 @@ def cpu_baseline(logits, ids, sample_rows: int):
         "kind": "port",
         "sample": f"{rows} of {total_rows} tokens ({n_blocks} blocks of {blk} rows, fp32 torch CPU "
                   f"log_softmax+gather), {elapsed:.1f} s; host cpu_count={os.cpu_count()}",
+        "parity": {"rows_compared": rows, "max_abs_err": max_err, "spike_rows": spike_rows,
+                   "spike_rows_with_target_on_spike": spike_hits, "spike_rows_max_abs_err": spike_err,
+                   "tolerance": PARITY_TOL, "ok": max_err <= PARITY_TOL},
     }
 
 
@@ -88,7 +116,7 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
         if batch == 256:
             gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                               "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel": "sample_rows<Bf16>"}
+                               "frac": gbps / HBM_PEAK_GBPS, **traffic_fields("sample_rows"), "kernel": "sample_rows<Bf16>"}
             # the other filter combinations at the same batch (kernel time per call, microseconds)
             modes = {}
             for name, kw in (("no_filter_T1", dict(temperature=1.0)), ("no_filter_T0.7", dict(temperature=0.7)),
@@ -152,7 +180,8 @@ def backward_throughput(sampler, iters: int = 5):
     return {"config": "bf16 logits [64,512,128256], gradient written in place; 4*V + 16 bytes per token",
             "ms": ms, "tokens_per_s": n / (ms * 1e-3),
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel": "logprob_backward_rows<Bf16,256,4,vec>"}}
+                         "frac": gbps / HBM_PEAK_GBPS, **traffic_fields("logprob_backward_rows"),
+                         "kernel": "logprob_backward_rows<Bf16,256,4,vec>", "bytes_per_launch": 8192 * (4 * V + 16)}}
 
 
 def lmhead_throughput(sampler, iters: int = 3):
@@ -179,7 +208,7 @@ def lmhead_throughput(sampler, iters: int = 3):
     return {"config": "hidden bf16 [32768,4096] ~ N(0,1), W bf16 [128256,4096] ~ N(0,0.02^2), seed 0; logits never stored",
             "ms": ms, "tokens_per_s": n / (ms * 1e-3),
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s",
-                         "frac": tflops / 2500.0, "traffic": None, "kernel": "lmhead_partials"}}
+                         "frac": tflops / 2500.0, **traffic_fields("lmhead_partials"), "kernel": "lmhead_partials"}}
 
 
 def main() -> int:
@@ -234,6 +263,13 @@ def main() -> int:
     for _ in range(args.warmup):
         sampler.compute_logp(logits3, ids2, chunk_tokens=chunk)
     torch.cuda.synchronize()
+    # Device memory one call needs beyond what is resident before it (logits + ids): the [G, L] fp32 result and
+    # whatever the operator allocates on the way (nothing of the size of the logits).
+    resident = torch.cuda.memory_allocated(dev)
+    torch.cuda.reset_peak_memory_stats(dev)
+    sampler.compute_logp(logits3, ids2, chunk_tokens=chunk)
+    torch.cuda.synchronize()
+    extra_device_bytes = torch.cuda.max_memory_allocated(dev) - resident
 
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -269,16 +305,19 @@ def main() -> int:
                                "rows, ids uniform, seed 0", "chunk_tokens": chunk,
                    "launches_per_step": launches_per_step, "input_dtype": "bf16", "output_dtype": "f32"},
         "hbm_gbps": n_rows * BYTES_PER_TOKEN / (ms_per_step * 1e-3) / 1e9,
+        "extra_device_bytes": extra_device_bytes,
+        "resident_bytes": resident,
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS,
-                     "traffic": rows_per_launch * MEASURED_TRAFFIC_PER_TOKEN,
+                     "traffic": STATIC_TRAFFIC["logprob_rows"][0] * rows_per_launch / 8192,
+                     "traffic_source": traffic_fields("logprob_rows")["traffic_source"],
                      "kernel": "logprob_rows<Bf16,256,4,vec>", "launch_ms": launch_ms,
                      "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
     }
     assert bool(torch.isfinite(out).all()), "non-finite logprob in the timed run"
     if args.cpu_sample_rows > 0:
         log("timing the CPU oracle on a sample of the same tensor")
-        result["cpu_baseline"] = cpu_baseline(logits, ids, args.cpu_sample_rows)
+        result["cpu_baseline"] = cpu_baseline(logits, ids, out, args.cpu_sample_rows)
     del logits3, ids2, logits, ids
     torch.cuda.empty_cache()
     result["logprob_backward"] = backward_throughput(sampler)
@@ -286,6 +325,10 @@ def main() -> int:
     if not args.skip_lmhead:
         result["fused_lm_head"] = lmhead_throughput(sampler)
     print(json.dumps(result), flush=True)
+    parity = result.get("cpu_baseline", {}).get("parity")
+    if parity is not None and not parity["ok"]:
+        log(f"PARITY FAILURE: max |GPU - CPU oracle| = {parity['max_abs_err']:.3e} > {PARITY_TOL}")
+        return 1
     return 0
 
 

@@ -8,10 +8,19 @@ the pool holds only the small scratch buffers of the other kernels (sampling
 histograms, fused lm_head partials).  It is one arena, allocated once per device
 and handed out by a bump pointer; on a 288 GB MI355X the default 64 MiB is
 0.02 % of HBM and the hard limit stays at 0.5 GB.
+
+Sharing rule.  Operators take their scratch through ``lease``: the pool's lock is
+held from the reservation to the end of the launch, so two host threads never
+hold the same bytes, and every lease leaves an event on the stream it was used
+on.  A later lease on another stream first makes that stream wait for the event,
+so kernels of two streams never work in the arena at the same time (they run one
+after the other; results are those of sequential calls).
 """
 from __future__ import annotations
 
 import os
+import threading
+from contextlib import contextmanager
 
 import torch
 
@@ -34,6 +43,8 @@ class WorkspacePool:
         self.capacity = (capacity_bytes + ALIGN - 1) // ALIGN * ALIGN
         self._arenas: dict = {}  # device index -> uint8 tensor
         self._offset = 0
+        self._lock = threading.RLock()
+        self._last_use: dict = {}  # device index -> (raw stream handle, event recorded behind the last lease)
 
     def arena(self, device: torch.device) -> torch.Tensor:
         index = device.index if device.index is not None else torch.cuda.current_device()
@@ -59,6 +70,27 @@ class WorkspacePool:
             )
         self._offset = start + nbytes
         return self.arena(device)[start:start + nbytes]
+
+    @contextmanager
+    def lease(self, nbytes: int, device: torch.device):
+        """``with pool.lease(n, device) as ws:`` — a uint8 view of ``n`` bytes for kernels enqueued on the
+        device's current stream inside the block.  Safe across streams and host threads (see the module
+        docstring): the whole arena is taken, the previous user's stream is waited for, and the lock is
+        released only after this user's event is recorded."""
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        with self._lock:
+            self.reset()
+            view = self.reserve(nbytes, device)
+            stream = torch.cuda.current_stream(torch.device("cuda", index))
+            last = self._last_use.get(index)
+            if last is not None and last[0] != stream.cuda_stream:
+                stream.wait_event(last[1])
+            try:
+                yield view
+            finally:
+                event = last[1] if last is not None else torch.cuda.Event()
+                event.record(stream)
+                self._last_use[index] = (stream.cuda_stream, event)
 
     def allocated_bytes(self) -> int:
         return self.capacity * len(self._arenas)

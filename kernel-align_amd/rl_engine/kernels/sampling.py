@@ -8,6 +8,8 @@ nothing falls back to torch ops.
 """
 from __future__ import annotations
 
+from contextlib import contextmanager
+
 import torch
 import torch.nn as nn
 
@@ -71,6 +73,16 @@ class SamplerBackend(nn.Module):
         self._lib = _hip.load()
         self.pool = WorkspacePool(pool_bytes)
         logger.info_once(f"Loaded {self._lib.ka_version().decode()}")
+
+    @contextmanager
+    def _workspace(self, nbytes: int, device):
+        """Device pointer of `nbytes` of scratch for launches on the current stream (None for no bytes).  The
+        pool orders users of different streams and threads, so one SamplerBackend may be shared by them."""
+        if nbytes == 0:
+            yield None
+            return
+        with self.pool.lease(nbytes, device) as view:
+            yield view.data_ptr()
 
     # ------------------------------------------------------------------ logprob
     @torch.inference_mode()
@@ -291,11 +303,9 @@ class SamplerBackend(nn.Module):
         if batch == 0:
             return (out, logprob) if return_logprob else out
         ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
-        self.pool.reset()
-        ws = self.pool.reserve(ws_bytes, dev)
         row_stride = rows.stride(0) if batch > 1 else vocab
         extended = return_logprob or k_rows is not None or p_rows is not None or t_rows is not None
-        with torch.cuda.device(dev):
+        with torch.cuda.device(dev), self._workspace(ws_bytes, dev) as ws_ptr:
             stream = torch.cuda.current_stream().cuda_stream
             if extended:
                 fn_name = "ka_sample_ex"
@@ -303,12 +313,12 @@ class SamplerBackend(nn.Module):
                 status = self._lib.ka_sample_ex(
                     _DTYPE_CODE[logits.dtype], rows.data_ptr(), batch, vocab, row_stride, t, ptr(t_rows), k,
                     ptr(k_rows), p, ptr(p_rows), uniforms.data_ptr(), out.data_ptr(), ptr(logprob),
-                    ws.data_ptr(), ws_bytes, stream)
+                    ws_ptr, ws_bytes, stream)
             else:
                 fn_name = _SAMPLE_FN[logits.dtype]
                 status = getattr(self._lib, fn_name)(
                     rows.data_ptr(), batch, vocab, row_stride, t, k, p, uniforms.data_ptr(),
-                    out.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+                    out.data_ptr(), ws_ptr, ws_bytes, stream)
         _hip.check(status, fn_name)
         return (out, logprob) if return_logprob else out
 
@@ -353,11 +363,10 @@ class SamplerBackend(nn.Module):
             for start in range(0, n_rows, rows_per_call):
                 n = min(rows_per_call, n_rows - start)
                 ws_bytes = self._lib.ka_lmhead_workspace_bytes(n, hdim, vocab)
-                self.pool.reset()
-                ws = self.pool.reserve(ws_bytes, hidden.device)
-                status = self._lib.ka_lmhead_logprob_bf16(
-                    h2.data_ptr() + start * hdim * 2, w2.data_ptr(), ids.data_ptr() + start * 8,
-                    out.data_ptr() + start * 4, n, hdim, vocab, ws.data_ptr(), ws_bytes, stream)
+                with self._workspace(ws_bytes, hidden.device) as ws_ptr:
+                    status = self._lib.ka_lmhead_logprob_bf16(
+                        h2.data_ptr() + start * hdim * 2, w2.data_ptr(), ids.data_ptr() + start * 8,
+                        out.data_ptr() + start * 4, n, hdim, vocab, ws_ptr, ws_bytes, stream)
                 _hip.check(status, "ka_lmhead_logprob_bf16")
         return out.view(tuple(hidden.shape[:-1]))
 

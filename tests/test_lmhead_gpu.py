@@ -154,3 +154,45 @@ def test_rows_are_sliced_to_fit_a_small_workspace_pool(sampler):
     with pytest.raises(PoolExhausted):
         tiny.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
     assert torch.equal(tiny.fused_linear_logp(hidden[:64].cuda(), weight.cuda(), ids[:64].cuda()), base[:64])
+
+
+def test_one_backend_shared_by_two_streams_and_two_threads(sampler):
+    """Calls on different streams (and from different host threads) share the backend's one workspace arena: the
+    pool orders them, so each result equals the sequential call's bit for bit.  Two inputs whose partials
+    overlap in the arena; were the kernels of the two streams to run in it at once, one would fold the other's
+    partials."""
+    import threading
+
+    a = tuple(t.cuda() for t in make(2048, 512, 30000, seed=31))
+    b = tuple(t.cuda() for t in make(1792, 512, 30000, seed=32))
+    want_a, want_b = sampler.fused_linear_logp(*a), sampler.fused_linear_logp(*b)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for _ in range(3):
+        with torch.cuda.stream(s1):
+            got_a = sampler.fused_linear_logp(*a)
+        with torch.cuda.stream(s2):
+            got_b = sampler.fused_linear_logp(*b)
+        with torch.cuda.stream(s1):
+            got_a2 = sampler.fused_linear_logp(*a)
+        torch.cuda.synchronize()
+        assert torch.equal(got_a, want_a) and torch.equal(got_b, want_b) and torch.equal(got_a2, want_a)
+
+    results, errors = {}, []
+
+    def worker(name, args, stream):
+        try:
+            with torch.cuda.stream(stream):
+                outs = [sampler.fused_linear_logp(*args) for _ in range(4)]
+            stream.synchronize()
+            results[name] = outs
+        except Exception as exc:  # noqa: BLE001
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=("a", a, s1)), threading.Thread(target=worker, args=("b", b, s2))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert all(torch.equal(o, want_a) for o in results["a"]) and all(torch.equal(o, want_b) for o in results["b"])

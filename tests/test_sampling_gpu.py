@@ -145,6 +145,26 @@ def test_every_bf16_value_through_the_temperature_step(sampler):
         check_exact(sampler, rows, u, 300, 0.95, temp)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_temperature_rule_against_torch_division_on_the_device(dtype):
+    """The operator's temperature step is the true quotient round_dtype(float(x) / T) (what torch's CPU division
+    returns, which is the oracle the parity target names).  torch's own GPU division by a Python scalar multiplies
+    by the fp32 reciprocal instead.  At the BASELINE temperature (0.7) and at 1.3 / 0.01 / 0.9 the two rules agree
+    on every finite 16-bit pattern; at e.g. 0.6 they differ on about 1.5 % of the patterns, which is recorded
+    here so that a change of either side shows up."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    x = bits[torch.isfinite(bits.float())]
+    for temp in (0.7, 1.3, 0.01, 0.9):
+        on_device = (x.cuda() / temp).cpu().float()
+        assert torch.equal(on_device, exact.scale(x, temp)), temp
+    on_device = (x.cuda() / 0.6).cpu().float()
+    reciprocal = (x.float() * (torch.tensor(1.0) / torch.tensor(0.6))).to(dtype).float()
+    assert torch.equal(on_device, reciprocal)                          # the device rule, restated
+    differ = int((on_device != exact.scale(x, 0.6)).sum())
+    assert 0 < differ < 0.03 * x.numel()
+    assert torch.equal((x / 0.6).float(), exact.scale(x, 0.6))         # the oracle is the CPU quotient
+
+
 def test_bit_identical_across_runs_and_batch_splits(sampler):
     logits, u = cfg5_sampling(256)
     dl, du = logits.cuda(), u.cuda()
