@@ -18,8 +18,6 @@
 // (ka_sampling_topk.h), and for 16-bit dtypes the no-filter and dense-histogram paths (ka_sampling_dense.h).
 // For aligned fp32 rows outside the candidate list a variant of the kernel replaces the last pass by a draw
 // over shares of the row (ka_sampling_draw.h).
-#include <stdlib.h>
-
 #include "ka_sampling_common.h"
 #include "ka_sampling_dense.h"
 #include "ka_sampling_topk.h"
@@ -86,16 +84,20 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     const bool use_k = top_k > 0 && top_k < vocab;
     const bool use_p = top_p < 1.0f;
 
+    KA_STAMP(0);
     float u = uniforms[row];
     if (!(u >= 0.0f)) u = 0.0f;
     if (u >= 1.0f) u = __uint_as_float(0x3f7fffffu);
 
-    if (!RADIX_ONLY && use_k && top_k <= S_THREADS && !no_fast) {
+    // no_fast: bit 0 = take the general radix path, bit 1 = keep the top-k route block-wide (KA_SAMPLE_FLAG_*)
+    if (!RADIX_ONLY && use_k && top_k <= S_THREADS && !(no_fast & 1)) {
         if constexpr (!RADIX_ONLY) {
-            if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot)) return;
+            if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot,
+                             (no_fast & 2) != 0))
+                return;
         }
         __syncthreads();
-    } else if (!no_fast) {
+    } else if (!(no_fast & 1)) {
         if constexpr (DENSE && T::kBytes == 2) {
             bool done;
             if (!use_k && !use_p)
@@ -312,15 +314,9 @@ __global__ __launch_bounds__(256) void mass_fixed_kernel(const float *__restrict
     if (i < n) out[i] = weight_fix(d[i]);
 }
 
-// KA_SAMPLE_RADIX_ONLY=1 switches the top-k fast path off (the tests use it to run both paths on every case).
-inline bool force_radix_path() {
-    const char *e = getenv("KA_SAMPLE_RADIX_ONLY");
-    return e != nullptr && e[0] == '1';
-}
-
 template <typename T>
 int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride, const SampleParams &prm,
-           void *workspace, size_t workspace_bytes, void *hip_stream) {
+           void *workspace, size_t workspace_bytes, void *hip_stream, uint32_t flags = 0) {
     if (batch < 0) return fail(KA_ERR_BAD_ARG, "sample: batch %lld < 0", (long long)batch);
     if (batch == 0) return KA_OK;
     if (logits == nullptr || prm.uniforms == nullptr || prm.out_ids == nullptr)
@@ -340,7 +336,10 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
         return fail(KA_ERR_WORKSPACE, "sample: workspace of %zu B, need %zu B", workspace_bytes,
                     ka_sample_workspace_bytes(batch, vocab));
     const bool aligned = (reinterpret_cast<uintptr_t>(logits) % 16 == 0) && ((row_stride * T::kBytes) % 16 == 0);
-    const bool no_fast = force_radix_path();
+    if (flags & ~uint32_t(KA_SAMPLE_FLAG_GENERAL_PATH | KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK))
+        return fail(KA_ERR_BAD_ARG, "sample: unknown flag bits 0x%x", flags);
+    const bool no_fast = (flags & KA_SAMPLE_FLAG_GENERAL_PATH) != 0;
+    const int path_bits = int(flags & 3u);
     // The dense-histogram path needs 157 KB of LDS (one workgroup per CU).  It serves top-p without top-k,
     // top_k > 1024 and no filter at all on aligned 16-bit rows; with per-row parameters any row may need it.
     bool dense = false;
@@ -363,7 +362,7 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
         const bool k_fast = prm.top_k > 0 && prm.top_k < vocab && prm.top_k <= S_THREADS;
         if (aligned && !per_row && !k_fast) {
             hipLaunchKernelGGL((sample_rows<T, true>), dim3(unsigned(batch)), dim3(S_THREADS), 0, stream, lp, int(vocab),
-                               row_stride, prm, 1, no_fast ? 1 : 0);
+                               row_stride, prm, 1, path_bits);
             return check_hip(hipGetLastError(), "sample launch");
         }
     }
@@ -373,12 +372,12 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(DENSE_LDS_BYTES));
         if (rc != hipSuccess) return check_hip(rc, "sample: reserving LDS for the dense-histogram path");
         hipLaunchKernelGGL((sample_rows<T, true>), dim3(unsigned(batch)), dim3(S_THREADS), DENSE_LDS_BYTES, stream, lp,
-                           int(vocab), row_stride, prm, aligned ? 1 : 0, 0);
+                           int(vocab), row_stride, prm, aligned ? 1 : 0, path_bits & 2);
         return check_hip(hipGetLastError(), "sample launch");
       }
     }
     hipLaunchKernelGGL((sample_rows<T, false>), dim3(unsigned(batch)), dim3(S_THREADS), 0, stream, lp, int(vocab),
-                       row_stride, prm, aligned ? 1 : 0, no_fast ? 1 : 0);
+                       row_stride, prm, aligned ? 1 : 0, path_bits);
     return check_hip(hipGetLastError(), "sample launch");
 }
 
@@ -394,11 +393,11 @@ inline SampleParams scalar_params(float temperature, int32_t top_k, float top_p,
 }
 
 inline int launch_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
-                     const SampleParams &prm, void *workspace, size_t workspace_bytes, void *hip_stream) {
+                     const SampleParams &prm, void *workspace, size_t workspace_bytes, void *hip_stream, uint32_t flags) {
     switch (dtype) {
-        case KA_DTYPE_BF16: return launch<Bf16>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream);
-        case KA_DTYPE_F16: return launch<F16>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream);
-        case KA_DTYPE_F32: return launch<F32>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream);
+        case KA_DTYPE_BF16: return launch<Bf16>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream, flags);
+        case KA_DTYPE_F16: return launch<F16>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream, flags);
+        case KA_DTYPE_F32: return launch<F32>(logits, batch, vocab, row_stride, prm, workspace, workspace_bytes, hip_stream, flags);
         default: return fail(KA_ERR_BAD_ARG, "sample: unknown dtype code %d", dtype);
     }
 }
@@ -438,6 +437,12 @@ KA_EXPORT int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t
                               workspace_bytes, hip_stream);
 }
 
+#ifdef KA_SAMPLE_STAMPS
+KA_EXPORT int ka_debug_read_stamps(unsigned long long *host, int n) {
+    return int(hipMemcpyFromSymbol(host, HIP_SYMBOL(ka::ka_dbg_stamps), size_t(n) * 8, 0, hipMemcpyDeviceToHost));
+}
+#endif
+
 KA_EXPORT int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, void *hip_stream) {
     using namespace ka;
     if (n < 0) return fail(KA_ERR_BAD_ARG, "mass: n %lld < 0", (long long)n);
@@ -452,12 +457,12 @@ KA_EXPORT int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, voi
 KA_EXPORT int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                            float temperature, const float *temperature_rows, int32_t top_k,
                            const int32_t *top_k_rows, float top_p, const float *top_p_rows, const float *uniforms,
-                           int64_t *out_ids, float *out_logprob, void *workspace, size_t workspace_bytes,
-                           void *hip_stream) {
+                           int64_t *out_ids, float *out_logprob, uint32_t flags, void *workspace,
+                           size_t workspace_bytes, void *hip_stream) {
     ka::SampleParams p = ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids);
     p.temperature_rows = temperature_rows;
     p.top_k_rows = top_k_rows;
     p.top_p_rows = top_p_rows;
     p.out_logprob = out_logprob;
-    return ka::launch_ex(dtype, logits, batch, vocab, row_stride, p, workspace, workspace_bytes, hip_stream);
+    return ka::launch_ex(dtype, logits, batch, vocab, row_stride, p, workspace, workspace_bytes, hip_stream, flags);
 }

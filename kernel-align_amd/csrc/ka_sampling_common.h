@@ -8,6 +8,16 @@
 namespace ka {
 namespace {
 
+// Phase stamps for timing experiments (block 0, thread 0 writes the shader clock at named points).
+#ifdef KA_SAMPLE_STAMPS
+__device__ unsigned long long ka_dbg_stamps[16 * 16 + 32];  // [wavefront][point], then 32 free slots
+#define KA_STAMP(i_) do { if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) ka_dbg_stamps[(threadIdx.x >> 6) * 16 + (i_)] = __builtin_readcyclecounter(); } while (0)
+#define KA_DBG_SET(i_, v_) do { ka_dbg_stamps[256 + (i_)] = (unsigned long long)(v_); } while (0)
+#else
+#define KA_STAMP(i_) do { } while (0)
+#define KA_DBG_SET(i_, v_) do { } while (0)
+#endif
+
 constexpr int S_THREADS = 1024;
 constexpr int S_WAVES = S_THREADS / kWave;
 constexpr int BINS = 2048;
@@ -160,7 +170,7 @@ struct alignas(16) Shared {
     int best_rb;
     uint32_t max_key;
     int64_t hit;
-    uint32_t n_cand, pick_a, pick_b;
+    uint32_t n_cand, n_vec, cand_kmax, pick_a, pick_b;
     uint64_t pick_z;
     DenseScalars ds;  // scalars of the resident no-filter path
 };

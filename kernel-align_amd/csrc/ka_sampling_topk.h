@@ -20,24 +20,160 @@ namespace {
 // Returns false (having written nothing) when the candidates do not fit: the radix path then runs.
 // All integer decisions are the same function of the row as in the radix path.
 // ---------------------------------------------------------------------------
+
+// ---------------------------------------------------------------------------
+// Pieces of the short route (top_k <= SHORT_TOPK): after the read of the row, five block-wide barriers and a tail on
+// one wavefront instead of radix descents and block-wide scans.
+// ---------------------------------------------------------------------------
+constexpr int SHORT_TOPK = 64;    // largest top_k the short route serves
+constexpr int SHORT_GROUPS = 128; // the 1024 lane maxima are pooled into this many group maxima (8 lanes each)
+constexpr int SHORT_VECS = 128;   // candidate vectors the short route takes (128 * 8 elements = one per thread)
+constexpr int SHORT_CAND = 256;   // candidates its tail takes (four per lane of one wavefront)
+
+// Cross-lane moves inside a group of eight lanes (DPP: no LDS traffic): lane ^ 1, lane ^ 2, and 7 - lane.
+__device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)); }
+__device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)); }
+__device__ __forceinline__ uint32_t dpp_half_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)); }
+
+// Inclusive prefix sum of one 64-bit value per lane over the wavefront, by DPP row shifts and row broadcasts.
+// One step: lanes outside ROW_MASK, and lanes whose source lies outside the row, add 0.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint64_t scan_step_u64(uint64_t v) {
+    const uint32_t lo = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v)), CTRL, ROW_MASK, 0xf, true));
+    const uint32_t hi = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v >> 32)), CTRL, ROW_MASK, 0xf, true));
+    return v + ((uint64_t(hi) << 32) | lo);
+}
+__device__ __forceinline__ uint64_t wave_incl_scan_u64(uint64_t v) {
+    v = scan_step_u64<0x111, 0xf>(v);  // row_shr:1
+    v = scan_step_u64<0x112, 0xf>(v);  // row_shr:2
+    v = scan_step_u64<0x114, 0xf>(v);  // row_shr:4
+    v = scan_step_u64<0x118, 0xf>(v);  // row_shr:8
+    v = scan_step_u64<0x142, 0xa>(v);  // row_bcast:15 -> rows 1 and 3
+    v = scan_step_u64<0x143, 0xc>(v);  // row_bcast:31 -> rows 2 and 3
+    return v;
+}
+
+// Minimum of one value per lane over the wavefront, in every lane (DPP row shifts and broadcasts, then lane 63).
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint32_t min_step_u32(uint32_t v) {
+    const uint32_t o = uint32_t(__builtin_amdgcn_update_dpp(int(0xffffffffu), int(v), CTRL, ROW_MASK, 0xf, false));
+    return o < v ? o : v;
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+    v = min_step_u32<0x111, 0xf>(v);
+    v = min_step_u32<0x112, 0xf>(v);
+    v = min_step_u32<0x114, 0xf>(v);
+    v = min_step_u32<0x118, 0xf>(v);
+    v = min_step_u32<0x142, 0xa>(v);
+    v = min_step_u32<0x143, 0xc>(v);
+    return uint32_t(__builtin_amdgcn_readlane(int(v), kWave - 1));
+}
+
+// Where the short route keeps its lists in the candidate area of LDS once the candidates are ranked (step S5):
+//   sh.c.raw[r], sh.c.sidx[r], sh.c.w[r]   scaled key, index and integer mass of the candidate of rank r, ranks by
+//                                           (key descending, index ascending);
+//   by_index_w(sh)[q], by_index_idx(sh)[q]  mass (0 until the tail files the kept ones) and index of the candidate
+//                                           that is q-th in ascending index order.
+__device__ __forceinline__ uint64_t *by_index_w(Shared &sh) { return sh.c.w + SHORT_CAND; }
+__device__ __forceinline__ uint32_t *by_index_idx(Shared &sh) { return reinterpret_cast<uint32_t *>(sh.c.w + 2 * SHORT_CAND); }
+
+// The tail of the short route on one wavefront, after the block has ranked the nc <= SHORT_CAND candidates both ways.
+// Position p of the key order is handled by slot p / 64 of lane p % 64; na <= 64 * SLOTS positions hold the top-k
+// survivors (ties kept).  Top-p cut on the prefix sums of the masses, then the kept masses are filed in index order
+// and a second prefix sum finds the first index whose inclusive mass exceeds floor(u * Z): the same integer decisions
+// as the block-wide tail, without a barrier and without a loop over pairs.
+template <typename T, int SLOTS>
+__device__ __forceinline__ void short_tail(Shared &sh, uint32_t nc, uint32_t na, const uint32_t *rank_by_index,
+                                           bool use_p, float top_p, float u, int64_t *out_slot, float *lp_slot) {
+    const int lane = threadIdx.x & (kWave - 1);
+    uint64_t w[SLOTS], before[SLOTS];
+    uint64_t carry = 0;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+        const uint32_t p = uint32_t(s * kWave + lane);
+        w[s] = p < na ? sh.c.w[p] : 0ull;
+        const uint64_t inc = wave_incl_scan_u64(w[s]);
+        before[s] = carry + inc - w[s];
+        carry += (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc >> 32)), kWave - 1))) << 32) |
+                 uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc)), kWave - 1));
+    }
+    const uint64_t z_topk = carry;
+    KA_STAMP(6);   // prefix of the masses
+    // top-p: `before` is non-decreasing along the key order, so the kept entries are a prefix; its mass is the
+    // inclusive sum at its last position.  Kept masses go to their place in index order.
+    uint64_t z_kept = 0;
+    {
+        const uint64_t theta = use_p ? floor_scale(top_p, z_topk) : ~0ull;
+        uint64_t *const wq = by_index_w(sh);
+#pragma unroll
+        for (int s = 0; s < SLOTS; ++s) {
+            const uint32_t p = uint32_t(s * kWave + lane);
+            const bool kept = p < na && before[s] <= theta;
+            const int n_here = __popcll(__ballot(kept));
+            if (n_here > 0) {
+                const uint64_t upto = before[s] + w[s];
+                z_kept = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(upto >> 32)), n_here - 1))) << 32) |
+                         uint32_t(__builtin_amdgcn_readlane(int(uint32_t(upto)), n_here - 1));
+            }
+            if (kept) wq[rank_by_index[p]] = w[s];
+        }
+    }
+    KA_STAMP(7);   // top-p cut
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // draw: inclusive mass in index order; the first position above floor(u * Z) wins
+    const uint64_t tau = floor_scale(u, z_kept);
+    uint32_t hit = 0xffffffffu;
+    uint64_t w_hit = 0;
+    {
+        const uint64_t *const wq = by_index_w(sh);
+        const uint32_t *const iq = by_index_idx(sh);
+        uint64_t base = 0;
+        for (uint32_t q0 = 0; q0 < nc; q0 += kWave) {  // wavefront-uniform: one to four rounds
+            const uint32_t q = q0 + uint32_t(lane);
+            const uint64_t wv = q < nc ? wq[q] : 0ull;
+            const uint64_t inc = base + wave_incl_scan_u64(wv);
+            const uint64_t above = __ballot(inc > tau);
+            if (above != 0) {
+                const int first = __ffsll((long long)above) - 1;
+                hit = iq[q0 + uint32_t(first)];
+                w_hit = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(wv >> 32)), first))) << 32) |
+                        uint32_t(__builtin_amdgcn_readlane(int(uint32_t(wv)), first));
+                break;
+            }
+            base = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc >> 32)), kWave - 1))) << 32) |
+                   uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc)), kWave - 1));
+        }
+    }
+    KA_STAMP(8);   // draw
+    if (lane == 0) {
+        *out_slot = hit == 0xffffffffu ? int64_t(-1) : int64_t(hit);
+        if (lp_slot != nullptr) *lp_slot = hit == 0xffffffffu ? __builtin_nanf("") : log_ratio(w_hit, z_kept);
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *rp, int vocab, bool vec, float temp,
                                           bool has_t, int top_k, bool use_p, float top_p, float u,
-                                          int64_t *out_slot, float *lp_slot) {
+                                          int64_t *out_slot, float *lp_slot, bool block_wide_only) {
     const int tid = threadIdx.x;
+    // top_k <= 64 takes the short route unless the caller asks for the block-wide one (the two give the same ids)
+    const bool short_route = top_k <= SHORT_TOPK && !block_wide_only;
     // 1. lane maxima of the raw values (float max: one convert and half a v_max3 per element; which of
     //    -0 / +0 it returns does not matter, any lower bound of the top_k-th element will do)
-    //    When the row fits (16-byte aligned, at most 16 vectors per lane: 131,072 bf16 entries) it is kept in
-    //    registers, so that the collection pass below reads nothing from memory.
+    //    On the block-wide route a row that fits (16-byte aligned, at most 16 vectors per lane: 131,072 bf16 entries)
+    //    is kept in registers, so that the collection pass below reads nothing from memory.  The short route keeps
+    //    32 maxima per lane instead and re-reads the few vectors that hold a candidate from L2: with 64 of a lane's
+    //    128 registers holding the row, its selection code spills, and the spills cost more than the re-reads.
     constexpr int EPV = T::kPerVec;
     constexpr int RES_VECS = 16;
     const int nvec = vocab / EPV;
-    const bool resident = vec && T::kDtype == KA_DTYPE_BF16 && nvec <= RES_VECS * S_THREADS;
+    const bool resident = !short_route && vec && T::kDtype == KA_DTYPE_BF16 && nvec <= RES_VECS * S_THREADS;
     // A longer or wider row does not fit in registers, but 32 maxima per lane do: slot r keeps the maximum of the
     // lane's vectors tid + (g * 32 + r) * 1024, g = 0 .. trk_rounds - 1, and the collection pass re-reads only the
     // slots that hold a candidate.  One vector per slot covers an fp32 row of 131,072 entries and a 16-bit row of
     // 262,144; longer fp32 rows take up to four vectors per slot (for the 16-bit dtypes the count stays a
-    // compile-time 1, which keeps their kernels as they are).
+    // compile-time 1, which keeps their kernels as they are).  (A resident row keeps no per-vector maxima: with the
+    // row in 64 registers of the 128 a lane has, sixteen more spill and slow the read down.)
     constexpr int TRK_VECS = 32;
     const int trk_need = (nvec + TRK_VECS * S_THREADS - 1) / (TRK_VECS * S_THREADS);
     const int trk_rounds = T::kBytes == 4 ? trk_need : 1;
@@ -45,28 +181,38 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     uint4 held[RES_VECS];
     float vmaxs[TRK_VECS];
     float lmaxf = -__builtin_inff();
+    auto vector_max = [](const uint4 &q) {
+        const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+        float vm = T::widen(e[0]);
+#pragma unroll
+        for (int j = 1; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
+        return vm;
+    };
     if (tracked) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll 1
         for (int round = 0; round < trk_rounds; ++round) {
             const int base = tid + round * TRK_VECS * S_THREADS;
 #pragma unroll
-            for (int g = 0; g < TRK_VECS / 8; ++g) {
-                uint4 q[8];
+            for (int g = 0; g < TRK_VECS / 16; ++g) {  // sixteen loads in flight per lane
+                if ((round * TRK_VECS + g * 16) * S_THREADS >= nvec) {  // block-uniform: nothing of the row is left
+                    if (round == 0) {
 #pragma unroll
-                for (int s = 0; s < 8; ++s) {
-                    const int v = base + (g * 8 + s) * S_THREADS;
+                        for (int s = 0; s < 16; ++s) vmaxs[g * 16 + s] = -__builtin_inff();
+                    }
+                    continue;
+                }
+                uint4 q[16];
+#pragma unroll
+                for (int s = 0; s < 16; ++s) {
+                    const int v = base + (g * 16 + s) * S_THREADS;
                     q[s] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
                 }
 #pragma unroll
-                for (int s = 0; s < 8; ++s) {
+                for (int s = 0; s < 16; ++s) {
                     float vm = -__builtin_inff();
-                    if (base + (g * 8 + s) * S_THREADS < nvec) {
-                        const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q[s]);
-#pragma unroll
-                        for (int j = 0; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
-                    }
-                    vmaxs[g * 8 + s] = round == 0 ? vm : fmaxf(vmaxs[g * 8 + s], vm);
+                    if (base + (g * 16 + s) * S_THREADS < nvec) vm = vector_max(q[s]);
+                    vmaxs[g * 16 + s] = round == 0 ? vm : fmaxf(vmaxs[g * 16 + s], vm);
                     lmaxf = fmaxf(lmaxf, vm);
                 }
             }
@@ -93,9 +239,195 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     } else {
         for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) { lmaxf = fmaxf(lmaxf, T::widen(raw)); });
     }
+    KA_STAMP(1);   // row read, lane maxima known
+    // 2. (both routes) the bound is widened over the raw values that scale to the same value; false: a huge
+    //    temperature folds too many values together
+    auto widen_bound = [&](uint32_t &bound) {
+        if (!has_t) return true;
+        const uint32_t ty = elem_key<T>(raw_of_key<T>(bound), temp, true);
+        int guard = 0;
+        while (bound >= key_step<T>() && guard < 64) {
+            const uint32_t prev = bound - key_step<T>();
+            if (elem_key<T>(raw_of_key<T>(prev), temp, true) < ty) break;
+            bound = prev;
+            ++guard;
+        }
+        return guard < 64;
+    };
+    bool have_candidates = false;  // the short route has filled the candidate list but leaves the tail to the block
+    if (short_route) {
+        // S1. The lane maxima are pooled into 128 group maxima (eight neighbouring lanes each); the top_k-th largest
+        //     group maximum is a lower bound of the top_k-th largest element (each group maximum is a different
+        //     element), and with top_k well below 128 nearly as tight as the top_k-th largest lane maximum.
+        float gmax = lmaxf;
+        gmax = fmaxf(gmax, __uint_as_float(dpp_xor1(__float_as_uint(gmax))));
+        gmax = fmaxf(gmax, __uint_as_float(dpp_xor2(__float_as_uint(gmax))));
+        gmax = fmaxf(gmax, __uint_as_float(dpp_half_mirror(__float_as_uint(gmax))));
+        if ((tid & 7) == 0) sh.c.skey[tid >> 3] = __float_as_uint(gmax);
+        if (tid == 0) { sh.n_cand = 0; sh.n_vec = 0; sh.hit = -1; sh.cand_kmax = 0; }
+        __syncthreads();
+        // S2. Eight threads rank one group maximum among the 128 (descending, ties by position): sixteen compares
+        //     each, summed inside the group of eight lanes.  Exactly one maximum has rank top_k - 1.
+        {
+            const int v = tid >> 3, part = tid & 7;
+            const float x = __uint_as_float(sh.c.skey[v]);
+            const uint4 *others = reinterpret_cast<const uint4 *>(sh.c.skey + part * 16);
+            uint32_t cnt = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint4 o = others[q];
+                const uint32_t ow[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float of = __uint_as_float(ow[e]);
+                    const int j = part * 16 + q * 4 + e;
+                    cnt += (of > x || (of == x && j < v)) ? 1u : 0u;
+                }
+            }
+            cnt += dpp_xor1(cnt);
+            cnt += dpp_xor2(cnt);
+            cnt += dpp_half_mirror(cnt);
+            if (part == 0 && cnt == uint32_t(top_k - 1)) sh.max_key = __float_as_uint(x);
+        }
+        __syncthreads();
+        KA_STAMP(2);   // bound known
+        uint32_t bound = masked_key<T>(__uint_as_float(sh.max_key));
+        if (!widen_bound(bound)) return false;
+        KA_STAMP(3);   // bound widened
+        const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
+        // Fewer than top_k groups hold a number above -inf: the survivors may include -inf entries (and NaNs, which
+        // count as -inf but fail every float compare).  Leave such rows to the radix path.
+        if (boundf == -__builtin_inff()) return false;
+        // S3. Vectors that hold a candidate go to a list in LDS whole (one atomic per vector, nothing per element
+        //     in the wavefronts that hold the row); single elements (ragged tail, unaligned rows) go straight to the
+        //     candidate list with their scaled key.
+        uint4 *const cvec = reinterpret_cast<uint4 *>(sh.c.w);  // [SHORT_VECS] vectors ...
+        uint32_t *const cvidx = sh.c.sidx;                      // ... and their vector numbers
+        auto add_vector = [&](int v, const uint4 &q) {
+            const uint32_t slot = atomicAdd(&sh.n_vec, 1u);
+            if (slot < uint32_t(SHORT_VECS)) {
+                cvec[slot] = q;
+                cvidx[slot] = uint32_t(v);
+            }
+        };
+        auto add_element = [&](int i, typename T::raw_t raw) {
+            if (T::widen(raw) >= boundf) {
+                const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
+                if (slot < CAND_CAP) {
+                    const uint32_t key = elem_key<T>(raw, temp, has_t);
+                    sh.c.raw[slot] = uint32_t(raw);
+                    sh.c.idx[slot] = uint32_t(i);
+                    sh.c.skey[slot] = key;
+                    atomicMax(&sh.cand_kmax, key);  // the row maximum is a candidate: the largest candidate key is its key
+                }
+            }
+        };
+        if (tracked) {
+            // Slots whose maximum reaches the bound (about top_k of the 32,768 slots of a row do).  Every lane then
+            // works through its own hits, one per turn, so that the loads of a wavefront go out together: a lane
+            // rarely has more than one, and a wavefront takes as many turns as its busiest lane has hits.
+            const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+            uint32_t hits = 0;
+#pragma unroll
+            for (int r = 0; r < TRK_VECS; ++r) hits |= vmaxs[r] >= boundf ? 1u << r : 0u;
+            while (__any(hits != 0)) {
+                if (hits != 0) {
+                    const int r = __ffs(hits) - 1;
+                    hits &= hits - 1;
+                    for (int round = 0; round < trk_rounds; ++round) {
+                        const int v = tid + (round * TRK_VECS + r) * S_THREADS;
+                        if (v < nvec) {
+                            const uint4 q = vp[v];
+                            if (trk_rounds == 1 || vector_max(q) >= boundf) add_vector(v, q);
+                        }
+                    }
+                }
+            }
+            const int i = nvec * EPV + tid;
+            if (i < vocab) add_element(i, rp[i]);
+        } else {
+            for_each_raw<T, 8>(rp, vocab, vec, add_element);
+        }
+        __syncthreads();
+        KA_STAMP(4);   // candidate vectors collected
+        const uint32_t nv = sh.n_vec;
+        if (nv <= uint32_t(SHORT_VECS)) {
+            // S4. One thread per element of the listed vectors: those at or above the bound join the candidate list.
+            if (tid < int(nv) * EPV) {
+                const int vslot = tid / EPV, e = tid % EPV;
+                const typename T::raw_t raw = reinterpret_cast<const typename T::raw_t *>(cvec + vslot)[e];
+                add_element(int(cvidx[vslot]) * EPV + e, raw);
+            }
+            __syncthreads();
+            KA_STAMP(10);  // candidates expanded
+            const uint32_t nc = sh.n_cand;
+            if (nc > CAND_CAP) return false;
+            if (nc <= uint32_t(SHORT_CAND)) {
+                // S5. Four threads rank one candidate twice, by (scaled key descending, index ascending) and by index
+                //     alone, and file it under both ranks together with its integer mass (see by_index_w above; none
+                //     of the arrays written here is read in this step).
+                uint32_t *const rank_by_index = sh.c.raw + SHORT_CAND;  // [key rank] -> position in index order
+                {
+                    const uint32_t c = uint32_t(tid) >> 2, part = uint32_t(tid) & 3u;
+                    uint32_t ki = 0, ii = 0, cnt = 0, cnt_i = 0;
+                    if (c < nc) {
+                        ki = sh.c.skey[c];
+                        ii = sh.c.idx[c];
+                        // the four threads of a candidate take every fourth group of four entries (16-byte reads;
+                        // entries past nc are stale but inside the list and masked out below)
+                        const uint4 *k4 = reinterpret_cast<const uint4 *>(sh.c.skey);
+                        const uint4 *i4 = reinterpret_cast<const uint4 *>(sh.c.idx);
+                        for (uint32_t m = part; m * 4 < nc; m += 4) {
+                            const uint4 kq = k4[m], iq = i4[m];
+                            const uint32_t kk[4] = {kq.x, kq.y, kq.z, kq.w}, ik[4] = {iq.x, iq.y, iq.z, iq.w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const bool live = m * 4 + e < nc;
+                                cnt += (live && (kk[e] > ki || (kk[e] == ki && ik[e] < ii))) ? 1u : 0u;
+                                cnt_i += (live && ik[e] < ii) ? 1u : 0u;
+                            }
+                        }
+                    }
+                    cnt += dpp_xor1(cnt);
+                    cnt += dpp_xor2(cnt);
+                    cnt_i += dpp_xor1(cnt_i);
+                    cnt_i += dpp_xor2(cnt_i);
+                    if (c < nc && part == 0) {
+                        const uint32_t kmax = sh.cand_kmax;
+                        sh.c.raw[cnt] = ki;
+                        sh.c.sidx[cnt] = ii;
+                        sh.c.w[cnt] = weight_fix(ki == kmax ? 0.0f : value_of<T>(ki) - value_of<T>(kmax));
+                        rank_by_index[cnt] = cnt_i;
+                        by_index_w(sh)[cnt_i] = 0;
+                        by_index_idx(sh)[cnt_i] = ii;
+                    }
+                }
+                __syncthreads();
+                KA_STAMP(5);   // candidates sorted
+                if (tid < kWave) {  // one wavefront finishes the row; the others are done
+                    // entries behind the top-k survivors play no part: the tail is sized by their number
+                    const uint32_t kstar = sh.c.raw[top_k - 1];
+                    uint32_t na = 0;
+#pragma unroll
+                    for (int s = 0; s < SHORT_CAND / kWave; ++s) {
+                        const uint32_t pp = uint32_t(s * kWave + tid);
+                        na += uint32_t(__popcll(__ballot(pp < nc && sh.c.raw[pp] >= kstar)));
+                    }
+                    if (na <= uint32_t(kWave)) short_tail<T, 1>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
+                    else if (na <= uint32_t(2 * kWave)) short_tail<T, 2>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
+                    else short_tail<T, 4>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
+                    KA_STAMP(9);
+                }
+                return true;
+            }
+            have_candidates = true;  // more than 256 candidates (a large tie group): the block-wide tail ranks them
+        }
+        __syncthreads();  // too many candidate vectors: the block-wide route starts over with its exact bound
+    }
+    if (!have_candidates) {
+    uint32_t bound = 0;
     const uint32_t lmax = masked_key<T>(lmaxf);
     // the top_k-th largest of the 1024 lane maxima, by the same MSB-first descent over count histograms
-    uint32_t bound = 0;
     {
         uint32_t rank = uint32_t(top_k), prefix = 0;
         for (int level = 0; level < Round<T>::kLevels; ++level) {
@@ -116,18 +448,9 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     }
     if (tid == 0) { sh.n_cand = 0; sh.hit = -1; }
     __syncthreads();
-    // 2. widen the bound over the raw values that scale to the same value
-    if (has_t) {
-        const uint32_t ty = elem_key<T>(raw_of_key<T>(bound), temp, true);
-        int guard = 0;
-        while (bound >= key_step<T>() && guard < 64) {
-            const uint32_t prev = bound - key_step<T>();
-            if (elem_key<T>(raw_of_key<T>(prev), temp, true) < ty) break;
-            bound = prev;
-            ++guard;
-        }
-        if (guard == 64) return false;  // a huge temperature folds many values together: radix path
-    }
+    KA_STAMP(2);   // bound known
+    if (!widen_bound(bound)) return false;
+    KA_STAMP(3);   // bound widened
     const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
     // Fewer than top_k lanes hold a number above -inf: the survivors then include -inf entries (and NaNs,
     // which count as -inf but fail every float compare).  Leave such rows to the radix path.
@@ -141,24 +464,19 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
             }
         }
     };
-    if (resident) {
+    // (after a fall-back from the short route the row is read again rather than kept in registers all the way here)
+    if (resident && !short_route) {
 #pragma unroll
         for (int r = 0; r < RES_VECS; ++r) {
-            const int v = tid + r * S_THREADS;
-            if (v < nvec) {
+            if (tid + r * S_THREADS < nvec && vector_max(held[r]) >= boundf) {  // rare: about top_k vectors of the row hold a candidate
                 const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&held[r]);
-                float vm = T::widen(e[0]);
 #pragma unroll
-                for (int j = 1; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
-                if (vm >= boundf) {  // rare: about top_k vectors of the whole row hold a candidate
-#pragma unroll
-                    for (int j = 0; j < EPV; ++j) collect(v * EPV + j, e[j]);
-                }
+                for (int j = 0; j < EPV; ++j) collect((tid + r * S_THREADS) * EPV + j, e[j]);
             }
         }
         const int i = nvec * EPV + tid;
         if (i < vocab) collect(i, rp[i]);
-    } else if (tracked) {
+    } else if (tracked && !short_route) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll
         for (int r = 0; r < TRK_VECS; ++r) {
@@ -180,6 +498,8 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         for_each_raw<T, 8>(rp, vocab, vec, collect);
     }
     __syncthreads();
+    KA_STAMP(4);   // candidates collected
+    }
     const uint32_t nc = sh.n_cand;
     if (nc > CAND_CAP) return false;
     // 3a. scale the candidates and rank them by (key desc, index asc)
@@ -223,6 +543,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         sh.c.sidx[rank] = my_idx;
     }
     __syncthreads();
+    KA_STAMP(5);
     // 3b. top-k with ties: survivors are the sorted prefix with key >= key of position top_k - 1
     const uint32_t kmax = sh.c.skey[0];
     const float vmax = value_of<T>(kmax);
@@ -256,6 +577,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         nb = sh.pick_a;
         z_kept = sh.pick_z;
     }
+    KA_STAMP(7);
     // 3d. draw: inclusive mass over the survivors in index order; the first index above floor(u * Z) wins
     const uint64_t tau = floor_scale(u, z_kept);
     if (tid < int(nb)) {
@@ -265,6 +587,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         if (cum > tau) atomicMin(reinterpret_cast<unsigned long long *>(&sh.hit), (unsigned long long)mine);
     }
     __syncthreads();
+    KA_STAMP(9);
     if (tid == 0) *out_slot = sh.hit;
     if (lp_slot != nullptr && tid < int(nb) && int64_t(sh.c.sidx[tid]) == sh.hit) *lp_slot = log_ratio(sh.c.w[tid], z_kept);
     return true;

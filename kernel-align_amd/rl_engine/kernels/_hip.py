@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint32, c_void_p
 from pathlib import Path
 
 KA_OK = 0
@@ -46,7 +46,7 @@ SIGNATURES = {
     "ka_sample_topk_topp_f16": (c_int, _SAMPLE_ARGS),
     "ka_sample_topk_topp_f32": (c_int, _SAMPLE_ARGS),
     "ka_sample_ex": (c_int, [c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_int32, c_void_p, c_float,
-                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+                             c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_size_t, c_void_p]),
     "ka_sample_mass_fixed": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "ka_lmhead_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "ka_lmhead_logprob_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
@@ -54,6 +54,10 @@ SIGNATURES = {
     "ka_lmhead_logprob_bf16_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                                c_void_p]),
 }
+
+# Route selection flags of ka_sample_ex (verification only; results do not depend on them).
+SAMPLE_FLAG_GENERAL_PATH = 1
+SAMPLE_FLAG_BLOCK_WIDE_TOPK = 2
 
 # Size of the static device array behind ka_lmhead_logprob_bf16_noalloc (KA_LMHEAD_STATIC_SCRATCH_BYTES).
 LMHEAD_STATIC_SCRATCH_BYTES = 16 << 20

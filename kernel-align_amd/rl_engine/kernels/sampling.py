@@ -244,7 +244,7 @@ class SamplerBackend(nn.Module):
     # ----------------------------------------------------------------- sampling
     @torch.inference_mode()
     def sample(self, logits, top_k=None, top_p=None, temperature=1.0, deterministic=True,
-               uniforms=None, generator=None, return_logprob=False):
+               uniforms=None, generator=None, return_logprob=False, route_flags=0):
         """Draw one token id per row after temperature -> top-k -> top-p filtering.
 
         logits: [B, V] bf16 / fp16 / fp32 on the GPU.  Returns int64 [B] (reference:
@@ -256,7 +256,8 @@ class SamplerBackend(nn.Module):
         ``top_k``, ``top_p`` and ``temperature`` may each be a [B] tensor of per-row values (a row value
         that is not valid switches that filter off for the row).  With ``return_logprob=True`` the result
         is ``(ids, logprob)`` where logprob (fp32 [B]) is the log-probability of the drawn token under the
-        filtered, renormalised distribution it was drawn from.
+        filtered, renormalised distribution it was drawn from.  ``route_flags`` (``_hip.SAMPLE_FLAG_*``) makes the
+        library take one of its slower routes for the same function; results do not depend on it.
         """
         _require_gpu(logits, "logits")
         if logits.dim() != 2:
@@ -304,7 +305,7 @@ class SamplerBackend(nn.Module):
             return (out, logprob) if return_logprob else out
         ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
         row_stride = rows.stride(0) if batch > 1 else vocab
-        extended = return_logprob or k_rows is not None or p_rows is not None or t_rows is not None
+        extended = return_logprob or k_rows is not None or p_rows is not None or t_rows is not None or route_flags
         with torch.cuda.device(dev), self._workspace(ws_bytes, dev) as ws_ptr:
             stream = torch.cuda.current_stream().cuda_stream
             if extended:
@@ -313,7 +314,7 @@ class SamplerBackend(nn.Module):
                 status = self._lib.ka_sample_ex(
                     _DTYPE_CODE[logits.dtype], rows.data_ptr(), batch, vocab, row_stride, t, ptr(t_rows), k,
                     ptr(k_rows), p, ptr(p_rows), uniforms.data_ptr(), out.data_ptr(), ptr(logprob),
-                    ws_ptr, ws_bytes, stream)
+                    int(route_flags), ws_ptr, ws_bytes, stream)
             else:
                 fn_name = _SAMPLE_FN[logits.dtype]
                 status = getattr(self._lib, fn_name)(

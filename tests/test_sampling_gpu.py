@@ -12,13 +12,18 @@ import torch
 
 from benchmarks.workloads import cfg5_sampling
 from oracle import exact, sampling_ref
+from rl_engine.kernels import _hip
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.bfloat16, torch.float16, torch.float32]
 
 
-def run(sampler, logits, u, k, p, temp):
-    return sampler.sample(logits.cuda(), top_k=k, top_p=p, temperature=temp, uniforms=u.cuda()).cpu()
+def run(sampler, logits, u, k, p, temp, route_flags=0):
+    return sampler.sample(logits.cuda(), top_k=k, top_p=p, temperature=temp, uniforms=u.cuda(),
+                          route_flags=route_flags).cpu()
+
+
+ROUTES = (0, _hip.SAMPLE_FLAG_BLOCK_WIDE_TOPK, _hip.SAMPLE_FLAG_GENERAL_PATH)   # shortest, block-wide top-k, radix
 
 
 def check_exact(sampler, logits, u, k, p, temp):
@@ -203,9 +208,10 @@ def test_invalid_arguments_raise(sampler):
         sampler.sample(logits, uniforms=torch.zeros(3, device="cuda"))
 
 
-def test_fast_and_radix_paths_are_the_same_function(sampler, monkeypatch):
-    """top_k <= 1024 normally runs on a candidate list in LDS; KA_SAMPLE_RADIX_ONLY=1 forces the radix
-    descents.  Both must return the same ids (and both are checked against the oracle elsewhere)."""
+def test_fast_and_radix_paths_are_the_same_function(sampler):
+    """top_k <= 1024 normally runs on a candidate list in LDS (for top_k <= 64 with wavefront-local sorts and a
+    one-wavefront tail, else block-wide); the route flags force the block-wide variant and the radix descents.
+    All must return the same ids (and each is checked against the oracle)."""
     g = torch.Generator().manual_seed(31)
     cases = []
     for dtype in DTYPES:
@@ -215,13 +221,46 @@ def test_fast_and_radix_paths_are_the_same_function(sampler, monkeypatch):
         cases.append((torch.zeros(4, 128256).to(dtype), 50, 0.3, 0.7))                                  # overflow -> radix
     for logits, k, p, temp in cases:
         u = torch.rand(logits.shape[0], generator=g)
-        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
-        fast = run(sampler, logits, u, k, p, temp)
-        monkeypatch.setenv("KA_SAMPLE_RADIX_ONLY", "1")
-        radix = run(sampler, logits, u, k, p, temp)
-        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
-        assert torch.equal(fast, radix)
+        fast, block, radix = (run(sampler, logits, u, k, p, temp, f) for f in ROUTES)
+        assert torch.equal(fast, radix) and torch.equal(fast, block)
         assert torch.equal(fast, exact.sample(logits, temp, k, p, u))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wavefront_route_of_small_top_k(sampler, dtype):
+    """top_k <= 64 bounds the candidates from per-wavefront sorted lane maxima and finishes on one wavefront with
+    1, 2 or 4 candidates per lane; beyond 256 candidates, or with top_k = 65, the block-wide tail takes over.
+    Rows are built to hit each of those sizes: smooth rows (few candidates), coarse grids (tie groups of tens to
+    hundreds of entries at the k-th value), a cut inside a tie group, the largest values packed into the share of
+    one lane / one wavefront (loose bounds), and all three routes must give the oracle's ids and log-probabilities."""
+    g = torch.Generator().manual_seed(77)
+    vocab = 40000
+    smooth = (torch.randn(16, vocab, generator=g) * 3)
+    coarse = (torch.randn(16, vocab, generator=g) * 3 * 2).round() / 2        # ~90 entries per value near the top
+    coarser = (torch.randn(16, vocab, generator=g) * 2).round()               # hundreds per value: above 256 candidates
+    packed = torch.randn(16, vocab, generator=g)
+    packed[:, :8 * 40] += 6.0                                                 # the top values sit in the vectors of 40 lanes
+    packed[8:, 8 * 64 * 3:8 * 64 * 4] += 9.0                                  # ... and in one wavefront's lanes
+    flat = torch.zeros(4, vocab)
+    flat[:, 5::97] = 1.0                                                      # 413 entries tie at the maximum
+    for rows, temps in ((smooth, (0.7, 1.0)), (coarse, (1.0, 0.5)), (coarser, (1.0,)), (packed, (0.7,)), (flat, (1.0,))):
+        logits = rows.to(dtype)
+        u = torch.rand(logits.shape[0], generator=g)
+        for k in (1, 2, 17, 50, 63, 64, 65):
+            for p in (None, 0.9, 0.3):
+                for temp in temps:
+                    want, want_lp = exact.sample_rows(logits, temp, k, p, u)
+                    for flags in ROUTES:
+                        ids, lp = sampler.sample(logits.cuda(), top_k=k, top_p=p, temperature=temp, uniforms=u.cuda(),
+                                                 return_logprob=True, route_flags=flags)
+                        assert torch.equal(ids.cpu(), want), (k, p, temp, flags)
+                        assert (lp.cpu().double() - want_lp).abs().max().item() < 1e-5
+
+
+def test_unknown_route_flag_is_refused(sampler):
+    logits, u = cfg5_sampling(4, vocab=1000)
+    with pytest.raises(ValueError, match="flag"):
+        sampler.sample(logits.cuda(), top_k=5, uniforms=u.cuda(), route_flags=8)
 
 
 def test_huge_temperature_folds_values_together(sampler):
@@ -233,7 +272,7 @@ def test_huge_temperature_folds_values_together(sampler):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_per_row_parameters_and_sampled_logprob(sampler, dtype, monkeypatch):
+def test_per_row_parameters_and_sampled_logprob(sampler, dtype):
     g = torch.Generator().manual_seed(41)
     batch, vocab = 40, 20000
     logits = (torch.randn(batch, vocab, generator=g) * 3).to(dtype)
@@ -246,12 +285,9 @@ def test_per_row_parameters_and_sampled_logprob(sampler, dtype, monkeypatch):
     ts = (torch.rand(batch, generator=g) * 1.5 + 0.3)
     ts[6], ts[7] = 1.0, -2.0                                              # identity, invalid -> 1
     want_ids, want_lp = exact.sample_rows(logits, ts, ks, ps, u)
-    for radix_only in (False, True):
-        if radix_only:
-            monkeypatch.setenv("KA_SAMPLE_RADIX_ONLY", "1")
+    for flags in ROUTES:
         ids, lp = sampler.sample(logits.cuda(), top_k=ks.cuda(), top_p=ps.cuda(), temperature=ts.cuda(),
-                                 uniforms=u.cuda(), return_logprob=True)
-        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
+                                 uniforms=u.cuda(), return_logprob=True, route_flags=flags)
         assert torch.equal(ids.cpu(), want_ids)
         assert (lp.cpu().double() - want_lp).abs().max().item() < 1e-5
         assert (lp <= 0).all()
@@ -269,7 +305,7 @@ def test_per_row_parameters_and_sampled_logprob(sampler, dtype, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_nan_and_infinite_logits_on_both_paths(sampler, dtype, monkeypatch):
+def test_nan_and_infinite_logits_on_both_paths(sampler, dtype):
     """NaN counts as -inf, +inf takes all the mass, rows with fewer than top_k numbers above -inf keep their
     -inf entries: same ids from the candidate-list path, the radix path and the oracle."""
     g = torch.Generator().manual_seed(43)
@@ -288,11 +324,9 @@ def test_nan_and_infinite_logits_on_both_paths(sampler, dtype, monkeypatch):
                                (allnan, 50, 0.9, 0.7)]:
         uu = u[:logits.shape[0]]
         want = exact.sample(logits, temp, k, p, uu)
-        for radix_only in ("0", "1"):
-            monkeypatch.setenv("KA_SAMPLE_RADIX_ONLY", radix_only)
-            got = run(sampler, logits, uu, k, p, temp)
-            assert torch.equal(got, want), f"radix_only={radix_only} k={k} p={p} T={temp}"
-        monkeypatch.delenv("KA_SAMPLE_RADIX_ONLY", raising=False)
+        for flags in ROUTES:
+            got = run(sampler, logits, uu, k, p, temp, flags)
+            assert torch.equal(got, want), f"route_flags={flags} k={k} p={p} T={temp}"
 
 
 def test_mass_function_is_bit_exact_against_the_oracle(sampler):
