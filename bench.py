@@ -181,7 +181,7 @@ def backward_throughput(sampler, iters: int = 5):
             "ms": ms, "tokens_per_s": n / (ms * 1e-3),
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": gbps / HBM_PEAK_GBPS, **traffic_fields("logprob_backward_rows"),
-                         "kernel": "logprob_backward_rows<Bf16,256,4,vec>", "bytes_per_launch": 8192 * (4 * V + 16)}}
+                         "kernel": "logprob_backward_rows<Bf16,1024,4,vec>", "bytes_per_launch": 8192 * (4 * V + 16)}}
 
 
 def lmhead_throughput(sampler, iters: int = 3):

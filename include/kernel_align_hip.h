@@ -194,6 +194,15 @@ int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t
                            size_t workspace_bytes, void *hip_stream);
 
 /*
+ * ka_lmhead_logprob_bf16 that also returns the entropy of every row's softmax over the vocabulary,
+ * entropy[r] = -sum_v p_v log p_v (fp32), from the same pass: one more accumulator per token in the kernel
+ * (about 1 % more time), same workspace.  No counterpart in the reference; GRPO-style losses consume both.
+ */
+int ka_lmhead_logprob_entropy_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                   float *entropy, int64_t n_rows, int64_t hidden_dim, int64_t vocab,
+                                   void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/*
  * ka_lmhead_logprob_bf16 for callers that cannot allocate device memory or bring a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same kernels, same results bit
  * for bit; the per-split partials go to a static array in device memory (KA_LMHEAD_STATIC_SCRATCH_BYTES,

@@ -39,7 +39,7 @@ constexpr int LM_BN = 256;      // tokens per workgroup
 constexpr int LM_BK = 64;       // hidden slab: one 128-byte line per row
 constexpr int LM_STAGES = 2;    // LDS: the slab in use and the slab in flight
 constexpr int LM_STAGE_ELEMS = (LM_BM + LM_BN) * LM_BK;  // bf16 elements per LDS stage (64 KB)
-constexpr int LM_XCH_BYTES = 2 * 4 * 32 * 3 * 4;  // exchange area of the end-of-item fold: [wave_n][tn][32 lanes][3 floats]
+constexpr int LM_XCH_BYTES = 2 * 4 * 32 * 4 * 4;  // exchange area of the end-of-item fold: [wave_n][tn][32 lanes][4 floats]
 constexpr int LM_LDS_BYTES = LM_STAGES * LM_STAGE_ELEMS * 2 + LM_XCH_BYTES;
 constexpr int LM_THREADS = 256;
 // Vocabulary tiles per split (at most).  Short splits let a single token block occupy many CUs: at
@@ -179,7 +179,7 @@ struct Partial {
     float m;   // max logit seen (>= kFloor)
     float s;   // sum of exp(logit - m)
     float xt;  // target logit if this split holds it, else -inf
-    float pad;
+    float pad; // ENTROPY: sum of x * exp(x - m), else 0
 };
 
 // LDS slab: 256 rows x 64 bf16 (128 B per row = eight 16-byte chunks).  A fragment read (ds_read_b128) has
@@ -192,7 +192,9 @@ typedef __attribute__((address_space(3))) void lds_void;
 
 // WIDE: a matrix of 4 GiB or more.  Hidden rows are then addressed relative to the cursor's token block and W rows by
 // 64-bit offsets; the ordinary kernel keeps 32-bit offsets from the two base pointers, which is 1 - 2 % faster.
-template <bool WIDE>
+// ENTROPY: also accumulate sum(x * exp(x - max)) per token (one more FMA per logit), from which the fold derives the
+// entropy of the row's softmax; it goes out in the fourth field of the partial.
+template <bool WIDE, bool ENTROPY>
 __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
     Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_splits, int n_token_blocks,
@@ -222,6 +224,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     if (v >= n_virtual) return;
 
     float m_run[4], ml2_run[4], s_run[4], xt[4];  // ml2_run = m_run * log2(e), kept so that it is never recomputed
+    float a_run[4];                               // ENTROPY: sum of x * exp(x - m_run)
     int target[4];
 
     // Global -> LDS copies.  One global_load_lds_dwordx4 moves 16 B per lane to LDS base + 16 * lane,
@@ -358,6 +361,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         m_run[tn] = kFloor;
         ml2_run[tn] = kFloor * kLog2e;
         s_run[tn] = 0.0f;
+        a_run[tn] = 0.0f;
         xt[tn] = -__builtin_inff();
         const int n = tok0 + wave_n * 128 + tn * 32 + l32;
         int64_t id = -1;
@@ -453,7 +457,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             const bool mine = d >= 0 && d < 128 && ((d >> 2) & 1) == lhalf;
             const int want = mine ? (((d >> 5) << 4) | ((d & 31) >> 3 << 2) | (d & 3)) : -1;  // tm*16 + r
             float mn = m_run[tn];
-            float part[4];
+            float part[4], parta[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             // Wavefront-uniform choice: almost every tile lies inside the vocabulary and holds no lane's target,
             // and then needs neither the bounds select nor the capture compare per logit.
             if (limit >= 128 && !__any(mine)) {
@@ -467,6 +471,16 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                     float e[16];
 #pragma unroll
                     for (int r = 0; r < 16; ++r) e[r] = fast_exp2(fmaf(acc[tm][tn][r], kLog2e, -ml2f));
+                    if constexpr (ENTROPY) {  // logits inside the vocabulary are finite: no 0 * inf here
+                        float xe[16];
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) xe[r] = acc[tm][tn][r] * e[r];
+#pragma unroll
+                        for (int step = 1; step < 16; step <<= 1)
+#pragma unroll
+                            for (int r = 0; r + step < 16; r += 2 * step) xe[r] += xe[r + step];
+                        parta[tm] = xe[0];
+                    }
 #pragma unroll
                     for (int step = 1; step < 16; step <<= 1)
 #pragma unroll
@@ -486,10 +500,19 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
 #pragma unroll
                 for (int tm = 0; tm < 4; ++tm) {
                     float e[16];
+                    float xe[16];
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const float x = (tm * 32 + (r >> 2) * 8 + (r & 3) < limit) ? acc[tm][tn][r] : -__builtin_inff();
                         e[r] = fast_exp2(fmaf(x, kLog2e, -ml2s));
+                        if constexpr (ENTROPY) xe[r] = e[r] == 0.0f ? 0.0f : x * e[r];  // rows past the vocabulary: 0, not 0 * -inf
+                    }
+                    if constexpr (ENTROPY) {
+#pragma unroll
+                        for (int step = 1; step < 16; step <<= 1)
+#pragma unroll
+                            for (int r = 0; r + step < 16; r += 2 * step) xe[r] += xe[r + step];
+                        parta[tm] = xe[0];
                     }
 #pragma unroll
                     for (int step = 1; step < 16; step <<= 1)
@@ -503,6 +526,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             // FMA against ml2n and return the rounding residue of a 1e30-sized product instead of 0
             const float rescale = fast_exp2(ml2_run[tn] - ml2n);
             s_run[tn] = fmaf(s_run[tn], rescale, (part[0] + part[1]) + (part[2] + part[3]));
+            if constexpr (ENTROPY) a_run[tn] = fmaf(a_run[tn], rescale, (parta[0] + parta[1]) + (parta[2] + parta[3]));
             m_run[tn] = mn;
             ml2_run[tn] = ml2n;
         }
@@ -518,21 +542,28 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         const float mm = fmaxf(m_run[tn], om);
         const float lo_s = lhalf == 0 ? s_run[tn] : os, lo_m = lhalf == 0 ? m_run[tn] : om;
         const float hi_s = lhalf == 0 ? os : s_run[tn], hi_m = lhalf == 0 ? om : m_run[tn];
-        s_run[tn] = lo_s * fast_exp2((lo_m - mm) * kLog2e) + hi_s * fast_exp2((hi_m - mm) * kLog2e);
+        const float f_lo = fast_exp2((lo_m - mm) * kLog2e), f_hi = fast_exp2((hi_m - mm) * kLog2e);
+        s_run[tn] = lo_s * f_lo + hi_s * f_hi;
+        if constexpr (ENTROPY) {
+            const float oa = __shfl_xor(a_run[tn], 32, kWave);
+            const float lo_a = lhalf == 0 ? a_run[tn] : oa, hi_a = lhalf == 0 ? oa : a_run[tn];
+            a_run[tn] = lo_a * f_lo + hi_a * f_hi;
+        }
         m_run[tn] = mm;
         xt[tn] = fmaxf(xt[tn], ox);
     }
     // ---- fold the two vocabulary halves of the tile through LDS (upper half -> lower half) ----
     // The exchange area lies behind the two stages, which already receive the first slabs of the next item.
     // One barrier is enough: the area is written again only after the next item's slabs, each with a barrier.
-    float *xch = reinterpret_cast<float *>(lds + LM_STAGES * LM_STAGE_ELEMS);  // [wave_n][tn][32][3]
+    float *xch = reinterpret_cast<float *>(lds + LM_STAGES * LM_STAGE_ELEMS);  // [wave_n][tn][32][4]
     if (wave_m == 1 && lhalf == 0) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
-            float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 3;
+            float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 4;
             p[0] = m_run[tn];
             p[1] = s_run[tn];
             p[2] = xt[tn];
+            if constexpr (ENTROPY) p[3] = a_run[tn];
         }
     }
     asm volatile("" ::: "memory");
@@ -542,10 +573,11 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     if (wave_m == 0 && lhalf == 0) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
-            const float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 3;
+            const float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 4;
             const float om = p[0], os = p[1], ox = p[2];
             const float mm = fmaxf(m_run[tn], om);
-            const float s = s_run[tn] * fast_exp2((m_run[tn] - mm) * kLog2e) + os * fast_exp2((om - mm) * kLog2e);
+            const float f_own = fast_exp2((m_run[tn] - mm) * kLog2e), f_other = fast_exp2((om - mm) * kLog2e);
+            const float s = s_run[tn] * f_own + os * f_other;
             const int n = tok0 + wave_n * 128 + tn * 32 + l32;
             if (n < n_rows) {
                 Partial out;
@@ -553,6 +585,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                 out.s = s;
                 out.xt = fmaxf(xt[tn], ox);
                 out.pad = 0.0f;
+                if constexpr (ENTROPY) out.pad = a_run[tn] * f_own + p[3] * f_other;
                 partials[size_t(sp) * n_rows + n] = out;
             }
         }
@@ -571,23 +604,26 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
 
 __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict__ partials,
                                                       const int64_t *__restrict__ ids, float *__restrict__ out,
-                                                      int n_rows, int vocab, int n_splits) {
+                                                      float *__restrict__ entropy, int n_rows, int vocab, int n_splits) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= n_rows) return;
     float mm = kFloor;
     for (int sp = 0; sp < n_splits; ++sp) mm = fmaxf(mm, partials[size_t(sp) * n_rows + n].m);
-    float s = 0.0f, x = -__builtin_inff();
+    float s = 0.0f, a = 0.0f, x = -__builtin_inff();
     for (int sp = 0; sp < n_splits; ++sp) {  // fixed split order
         const Partial p = partials[size_t(sp) * n_rows + n];
-        s += p.s * fast_exp2((p.m - mm) * kLog2e);
+        const float f = fast_exp2((p.m - mm) * kLog2e);
+        s += p.s * f;
+        a += p.pad * f;
         x = fmaxf(x, p.xt);
     }
+    const double lse = double(mm) + log2(double(s)) * kLn2;
+    if (entropy != nullptr) entropy[n] = float(lse - double(a) / double(s));  // -sum p log p = lse - sum p x
     const int64_t id = ids[n];
     if (id < 0 || id >= vocab) {
         out[n] = __builtin_nanf("");
         return;
     }
-    const double lse = double(mm) + log2(double(s)) * kLn2;
     out[n] = float(double(x) - lse);
 }
 
@@ -638,11 +674,12 @@ int lm_current_device(bool need_scratch, LmDevice &out) {
         rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
         if (rc != hipSuccess) return check_hip(rc, "lmhead: querying the CU count");
         // the attribute belongs to the device, so it is set once per device and not once per process
-        rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials<false>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
-        if (rc == hipSuccess)
-            rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials<true>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
+        const void *kernels[4] = {reinterpret_cast<const void *>(lmhead_partials<false, false>),
+                                  reinterpret_cast<const void *>(lmhead_partials<true, false>),
+                                  reinterpret_cast<const void *>(lmhead_partials<false, true>),
+                                  reinterpret_cast<const void *>(lmhead_partials<true, true>)};
+        for (int k = 0; k < 4 && rc == hipSuccess; ++k)
+            rc = hipFuncSetAttribute(kernels[k], hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
         if (rc != hipSuccess) return check_hip(rc, "lmhead: reserving 131 KB of LDS");
         d.cus = cus;
         d.ready = true;
@@ -676,7 +713,7 @@ int lm_check_args(const void *hidden, const void *weight, const int64_t *ids, co
 
 // Enqueues the two kernels; `partials` holds ka_lmhead_workspace_bytes(n_rows, ., vocab) bytes of device memory.
 int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const int64_t *ids, float *out,
-              int64_t n_rows, int64_t hidden_dim, int64_t vocab, Partial *partials, hipStream_t stream) {
+              float *entropy, int64_t n_rows, int64_t hidden_dim, int64_t vocab, Partial *partials, hipStream_t stream) {
     const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
     const int n_splits = splits_for(vocab);
     const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
@@ -687,28 +724,29 @@ int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const
     const int64_t resident = dev.cus >= 256 ? 256 : (dev.cus >= 8 ? dev.cus / 8 * 8 : 8);
     const int64_t grid = n_virtual < resident ? n_virtual : resident;
     const bool wide = n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32);
-    if (wide)
-        hipLaunchKernelGGL(lmhead_partials<true>, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                            static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
                            int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
-    else
-        hipLaunchKernelGGL(lmhead_partials<false>, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
-                           static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
-                           int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
+    };
+    if (entropy != nullptr) {
+        if (wide) launch(lmhead_partials<true, true>);
+        else launch(lmhead_partials<false, true>);
+    } else {
+        if (wide) launch(lmhead_partials<true, false>);
+        else launch(lmhead_partials<false, false>);
+    }
     int rc = check_hip(hipGetLastError(), "lmhead partials launch");
     if (rc != KA_OK) return rc;
     hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids, out,
-                       int(n_rows), int(vocab), n_splits);
+                       entropy, int(n_rows), int(vocab), n_splits);
     return check_hip(hipGetLastError(), "lmhead combine launch");
 }
 
-}  // namespace
-}  // namespace ka
-
-KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
-                                     int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
-                                     size_t workspace_bytes, void *hip_stream) {
-    using namespace ka;
+// Everything the workspace entry points share.
+int lm_with_workspace(const void *hidden, const void *weight, const int64_t *ids, float *out, float *entropy,
+                      int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace, size_t workspace_bytes,
+                      void *hip_stream) {
     if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead: n_rows %lld < 0", (long long)n_rows);
     if (n_rows == 0) return KA_OK;
     int rc = lm_check_args(hidden, weight, ids, out, n_rows, hidden_dim, vocab);
@@ -719,8 +757,26 @@ KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, con
     LmDevice dev;
     rc = lm_current_device(false, dev);
     if (rc != KA_OK) return rc;
-    return lm_launch(dev, hidden, weight, ids, out, n_rows, hidden_dim, vocab, static_cast<Partial *>(workspace),
+    return lm_launch(dev, hidden, weight, ids, out, entropy, n_rows, hidden_dim, vocab, static_cast<Partial *>(workspace),
                      static_cast<hipStream_t>(hip_stream));
+}
+
+}  // namespace
+}  // namespace ka
+
+KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                     int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
+                                     size_t workspace_bytes, void *hip_stream) {
+    return ka::lm_with_workspace(hidden, weight, ids, out, nullptr, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
+                                 hip_stream);
+}
+
+KA_EXPORT int ka_lmhead_logprob_entropy_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                             float *entropy, int64_t n_rows, int64_t hidden_dim, int64_t vocab,
+                                             void *workspace, size_t workspace_bytes, void *hip_stream) {
+    if (entropy == nullptr && n_rows > 0) return ka::fail(KA_ERR_BAD_ARG, "lmhead: null entropy pointer");
+    return ka::lm_with_workspace(hidden, weight, ids, out, entropy, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
+                                 hip_stream);
 }
 
 KA_EXPORT int ka_lmhead_logprob_bf16_noalloc(const void *hidden, const void *weight, const int64_t *ids, float *out,
@@ -740,6 +796,6 @@ KA_EXPORT int ka_lmhead_logprob_bf16_noalloc(const void *hidden, const void *wei
     rc = lm_current_device(true, dev);
     if (rc != KA_OK) return rc;
     // Nothing in the scratch has to start at zero: every partial the fold reads is written by this call's first kernel.
-    return lm_launch(dev, hidden, weight, ids, out, n_rows, hidden_dim, vocab, static_cast<Partial *>(dev.scratch),
+    return lm_launch(dev, hidden, weight, ids, out, nullptr, n_rows, hidden_dim, vocab, static_cast<Partial *>(dev.scratch),
                      static_cast<hipStream_t>(hip_stream));
 }

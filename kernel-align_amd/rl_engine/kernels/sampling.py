@@ -325,14 +325,15 @@ class SamplerBackend(nn.Module):
 
     # ---------------------------------------------------------------- fused GEMM
     @torch.inference_mode()
-    def fused_linear_logp(self, hidden, weight, token_ids):
-        return self._fused_linear_logp(hidden, weight, token_ids)
+    def fused_linear_logp(self, hidden, weight, token_ids, return_entropy=False):
+        return self._fused_linear_logp(hidden, weight, token_ids, return_entropy)
 
-    def _fused_linear_logp(self, hidden, weight, token_ids):
+    def _fused_linear_logp(self, hidden, weight, token_ids, return_entropy=False):
         """``compute_logp(hidden @ weight.T, token_ids)`` without materialising the logits.
 
         hidden: bf16 [..., H]; weight: bf16 [V, H] (nn.Linear.weight layout); token_ids: integer
-        tensor of shape hidden.shape[:-1].  Returns fp32 of that shape.
+        tensor of shape hidden.shape[:-1].  Returns fp32 of that shape; with ``return_entropy=True`` a pair
+        ``(logp, entropy)`` where entropy is that of each row's softmax over the vocabulary, from the same pass.
         """
         _require_gpu(hidden, "hidden")
         _require_gpu(weight, "weight")
@@ -349,8 +350,10 @@ class SamplerBackend(nn.Module):
         n_rows = h2.shape[0]
         ids = token_ids.to(device=hidden.device, dtype=torch.int64).contiguous().view(-1)
         out = torch.empty(n_rows, dtype=torch.float32, device=hidden.device)
+        ent = torch.empty(n_rows, dtype=torch.float32, device=hidden.device) if return_entropy else None
+        lead = tuple(hidden.shape[:-1])
         if n_rows == 0:
-            return out.view(tuple(hidden.shape[:-1]))
+            return (out.view(lead), ent.view(lead)) if return_entropy else out.view(lead)
         # The workspace holds 16 B per row and vocabulary split; rows go to the kernel in slices that fit
         # the pool (a multiple of the 256-token tile), which does not change any row's result.
         per_row = self._lib.ka_lmhead_workspace_bytes(256, hdim, vocab) // 256
@@ -365,11 +368,17 @@ class SamplerBackend(nn.Module):
                 n = min(rows_per_call, n_rows - start)
                 ws_bytes = self._lib.ka_lmhead_workspace_bytes(n, hdim, vocab)
                 with self._workspace(ws_bytes, hidden.device) as ws_ptr:
-                    status = self._lib.ka_lmhead_logprob_bf16(
-                        h2.data_ptr() + start * hdim * 2, w2.data_ptr(), ids.data_ptr() + start * 8,
-                        out.data_ptr() + start * 4, n, hdim, vocab, ws_ptr, ws_bytes, stream)
+                    if return_entropy:
+                        status = self._lib.ka_lmhead_logprob_entropy_bf16(
+                            h2.data_ptr() + start * hdim * 2, w2.data_ptr(), ids.data_ptr() + start * 8,
+                            out.data_ptr() + start * 4, ent.data_ptr() + start * 4, n, hdim, vocab, ws_ptr, ws_bytes,
+                            stream)
+                    else:
+                        status = self._lib.ka_lmhead_logprob_bf16(
+                            h2.data_ptr() + start * hdim * 2, w2.data_ptr(), ids.data_ptr() + start * 8,
+                            out.data_ptr() + start * 4, n, hdim, vocab, ws_ptr, ws_bytes, stream)
                 _hip.check(status, "ka_lmhead_logprob_bf16")
-        return out.view(tuple(hidden.shape[:-1]))
+        return (out.view(lead), ent.view(lead)) if return_entropy else out.view(lead)
 
     @torch.inference_mode()
     def fused_linear_logp_backward(self, hidden, weight, token_ids, grad_logp, chunk_tokens=None,

@@ -93,6 +93,10 @@ def test_lmhead_argument_checks_and_workspace_size():
     assert call(p, p, p, p, 4, 4096, 128256, None, 0, None) == _hip.KA_ERR_WORKSPACE
     assert call(p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
     assert b"workspace" in lib.ka_last_error()
+    ent = lib.ka_lmhead_logprob_entropy_bf16
+    assert ent(None, None, None, None, None, 0, 4096, 128256, None, 0, None) == _hip.KA_OK
+    assert ent(p, p, p, p, None, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG           # entropy missing
+    assert ent(p, p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
     # the variant without a workspace argument: same checks, and a size limit instead of a workspace check
     na = lib.ka_lmhead_logprob_bf16_noalloc
     assert na(None, None, None, None, 0, 4096, 128256, None) == _hip.KA_OK

@@ -196,3 +196,26 @@ def test_one_backend_shared_by_two_streams_and_two_threads(sampler):
         t.join()
     assert not errors, errors
     assert all(torch.equal(o, want_a) for o in results["a"]) and all(torch.equal(o, want_b) for o in results["b"])
+
+
+@pytest.mark.parametrize("n,h,v", [(5, 64, 7), (300, 256, 1000), (257, 192, 16129), (700, 512, 16385), (384, 4096, 128256)])
+def test_entropy_from_the_same_pass(sampler, n, h, v):
+    """fused_linear_logp(..., return_entropy=True): the log-probabilities are those of the plain call bit for bit
+    (the entropy accumulator does not touch the max / sum arithmetic), and the entropy matches the fp64 entropy of
+    softmax(hidden @ W^T) - ragged last tile and last token block included."""
+    hidden, weight, ids = make(n, h, v, seed=3 * n + v, w_scale=0.2 if v < 100000 else 0.02)
+    hg, wg, ig = hidden.cuda(), weight.cuda(), ids.cuda()
+    lp, ent = sampler.fused_linear_logp(hg, wg, ig, return_entropy=True)
+    assert torch.equal(lp, sampler.fused_linear_logp(hg, wg, ig))
+    assert ent.shape == (n,) and ent.dtype == torch.float32
+    if v > 100000:
+        logits = torch.nn.functional.linear(hidden[:64].double(), weight.double())
+        want = O.entropy_f64(logits)
+        assert (ent[:64].cpu().double() - want).abs().max().item() <= TOL
+        # and the unfused route on the device agrees on every row
+        lp2, ent2 = sampler.compute_logp_entropy(torch.nn.functional.linear(hg.float(), wg.float()), ig)
+        assert (ent - ent2).abs().max().item() <= TOL
+    else:
+        want = O.entropy_f64(torch.nn.functional.linear(hidden.double(), weight.double()))
+        assert (ent.cpu().double() - want).abs().max().item() <= TOL
+    assert (ent > 0).all() and (ent.cpu() <= math.log(v) + 1e-4).all()
