@@ -175,11 +175,38 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     // compile-time 1, which keeps their kernels as they are).  (A resident row keeps no per-vector maxima: with the
     // row in 64 registers of the 128 a lane has, sixteen more spill and slow the read down.)
     constexpr int TRK_VECS = 32;
+#ifndef KA_TRK_BATCH
+#define KA_TRK_BATCH 8
+#endif
+    constexpr int TRK_BATCH = KA_TRK_BATCH;  // loads in flight per lane (with 16, the 128 registers of a lane spill)
     const int trk_need = (nvec + TRK_VECS * S_THREADS - 1) / (TRK_VECS * S_THREADS);
     const int trk_rounds = T::kBytes == 4 ? trk_need : 1;
     const bool tracked = vec && !resident && trk_need <= (T::kBytes == 4 ? 4 : 1);
     uint4 held[RES_VECS];
-    float vmaxs[TRK_VECS];
+    // The slot maxima of a 16-bit row are kept in the row's own 16 bits, two per register (they are elements of the
+    // row, so nothing is lost): 32 floats next to the loads in flight would spill.
+    constexpr bool PACKED = T::kBytes == 2;
+    uint32_t vstore[PACKED ? TRK_VECS / 2 : TRK_VECS];
+    auto narrow16 = [](float v) -> uint32_t {
+        if (T::kDtype == KA_DTYPE_F16) {
+            union { _Float16 h; uint16_t u; } c;
+            c.h = _Float16(v);
+            return c.u;
+        }
+        return __float_as_uint(v) >> 16;
+    };
+    auto set_slot_max = [&](int slot, float vm, bool first_round) {  // slot is a compile-time value at every call
+        if (PACKED) {
+            if ((slot & 1) == 0) vstore[slot / 2] = narrow16(vm);
+            else vstore[slot / 2] |= narrow16(vm) << 16;
+        } else {
+            vstore[slot] = __float_as_uint(first_round ? vm : fmaxf(__uint_as_float(vstore[slot]), vm));
+        }
+    };
+    auto slot_max = [&](int slot) -> float {
+        if (PACKED) return T::widen(typename T::raw_t((slot & 1) == 0 ? (vstore[slot / 2] & 0xffffu) : (vstore[slot / 2] >> 16)));
+        return __uint_as_float(vstore[slot]);
+    };
     float lmaxf = -__builtin_inff();
     auto vector_max = [](const uint4 &q) {
         const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
@@ -194,25 +221,25 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         for (int round = 0; round < trk_rounds; ++round) {
             const int base = tid + round * TRK_VECS * S_THREADS;
 #pragma unroll
-            for (int g = 0; g < TRK_VECS / 16; ++g) {  // sixteen loads in flight per lane
-                if ((round * TRK_VECS + g * 16) * S_THREADS >= nvec) {  // block-uniform: nothing of the row is left
+            for (int g = 0; g < TRK_VECS / TRK_BATCH; ++g) {
+                if ((round * TRK_VECS + g * TRK_BATCH) * S_THREADS >= nvec) {  // block-uniform: nothing of the row is left
                     if (round == 0) {
 #pragma unroll
-                        for (int s = 0; s < 16; ++s) vmaxs[g * 16 + s] = -__builtin_inff();
+                        for (int s = 0; s < TRK_BATCH; ++s) set_slot_max(g * TRK_BATCH + s, -__builtin_inff(), true);
                     }
                     continue;
                 }
-                uint4 q[16];
+                uint4 q[TRK_BATCH];
 #pragma unroll
-                for (int s = 0; s < 16; ++s) {
-                    const int v = base + (g * 16 + s) * S_THREADS;
+                for (int s = 0; s < TRK_BATCH; ++s) {
+                    const int v = base + (g * TRK_BATCH + s) * S_THREADS;
                     q[s] = v < nvec ? vp[v] : make_uint4(0, 0, 0, 0);
                 }
 #pragma unroll
-                for (int s = 0; s < 16; ++s) {
+                for (int s = 0; s < TRK_BATCH; ++s) {
                     float vm = -__builtin_inff();
-                    if (base + (g * 16 + s) * S_THREADS < nvec) vm = vector_max(q[s]);
-                    vmaxs[g * 16 + s] = round == 0 ? vm : fmaxf(vmaxs[g * 16 + s], vm);
+                    if (base + (g * TRK_BATCH + s) * S_THREADS < nvec) vm = vector_max(q[s]);
+                    set_slot_max(g * TRK_BATCH + s, vm, round == 0);
                     lmaxf = fmaxf(lmaxf, vm);
                 }
             }
@@ -329,7 +356,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
             const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
             uint32_t hits = 0;
 #pragma unroll
-            for (int r = 0; r < TRK_VECS; ++r) hits |= vmaxs[r] >= boundf ? 1u << r : 0u;
+            for (int r = 0; r < TRK_VECS; ++r) hits |= slot_max(r) >= boundf ? 1u << r : 0u;
             while (__any(hits != 0)) {
                 if (hits != 0) {
                     const int r = __ffs(hits) - 1;
@@ -480,7 +507,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll
         for (int r = 0; r < TRK_VECS; ++r) {
-            if (vmaxs[r] >= boundf) {  // rare: about top_k slots of the whole row hold a candidate
+            if (slot_max(r) >= boundf) {  // rare: about top_k slots of the whole row hold a candidate
                 for (int round = 0; round < trk_rounds; ++round) {
                     const int v = tid + (round * TRK_VECS + r) * S_THREADS;
                     if (v < nvec) {
