@@ -2,6 +2,8 @@
 #ifndef KA_SAMPLING_TOPK_H
 #define KA_SAMPLING_TOPK_H
 
+#include <type_traits>
+
 #include "ka_sampling_common.h"
 
 namespace ka {
@@ -30,9 +32,11 @@ constexpr int SHORT_GROUPS = 128; // the 1024 lane maxima are pooled into this m
 constexpr int SHORT_VECS = 128;   // candidate vectors the short route takes (128 * 8 elements = one per thread)
 constexpr int SHORT_CAND = 256;   // candidates its tail takes (four per lane of one wavefront)
 
-// Cross-lane moves inside a group of eight lanes (DPP: no LDS traffic): lane ^ 1, lane ^ 2, and 7 - lane.
+// Cross-lane moves inside a row of sixteen lanes (DPP: no LDS traffic): lane ^ 1, lane ^ 2, 7 - lane inside each
+// half row, and 15 - lane.  Applied in this order, a sum (or maximum) over 2, 4, 8, 16 neighbouring lanes builds up.
 __device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)); }
 __device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)); }
+__device__ __forceinline__ uint32_t dpp_row_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)); }
 __device__ __forceinline__ uint32_t dpp_half_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)); }
 
 // Inclusive prefix sum of one 64-bit value per lane over the wavefront, by DPP row shifts and row broadcasts.
@@ -394,17 +398,20 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                 //     alone, and file it under both ranks together with its integer mass (see by_index_w above; none
                 //     of the arrays written here is read in this step).
                 uint32_t *const rank_by_index = sh.c.raw + SHORT_CAND;  // [key rank] -> position in index order
-                {
-                    const uint32_t c = uint32_t(tid) >> 2, part = uint32_t(tid) & 3u;
+                // PARTS threads share a candidate (16 for up to 64 candidates, 8 up to 128, 4 up to 256: all 1024
+                // threads take part), each over every PARTS-th group of four entries; the counts are summed inside the
+                // PARTS neighbouring lanes by DPP.
+                auto rank_candidates = [&](auto parts_c) {
+                    constexpr uint32_t PARTS = decltype(parts_c)::value;
+                    const uint32_t c = uint32_t(tid) / PARTS, part = uint32_t(tid) % PARTS;
                     uint32_t ki = 0, ii = 0, cnt = 0, cnt_i = 0;
                     if (c < nc) {
                         ki = sh.c.skey[c];
                         ii = sh.c.idx[c];
-                        // the four threads of a candidate take every fourth group of four entries (16-byte reads;
-                        // entries past nc are stale but inside the list and masked out below)
+                        // 16-byte reads; entries past nc are stale but inside the list and masked out below
                         const uint4 *k4 = reinterpret_cast<const uint4 *>(sh.c.skey);
                         const uint4 *i4 = reinterpret_cast<const uint4 *>(sh.c.idx);
-                        for (uint32_t m = part; m * 4 < nc; m += 4) {
+                        for (uint32_t m = part; m * 4 < nc; m += PARTS) {
                             const uint4 kq = k4[m], iq = i4[m];
                             const uint32_t kk[4] = {kq.x, kq.y, kq.z, kq.w}, ik[4] = {iq.x, iq.y, iq.z, iq.w};
 #pragma unroll
@@ -415,10 +422,13 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                             }
                         }
                     }
-                    cnt += dpp_xor1(cnt);
-                    cnt += dpp_xor2(cnt);
-                    cnt_i += dpp_xor1(cnt_i);
-                    cnt_i += dpp_xor2(cnt_i);
+                    uint32_t both = cnt | (cnt_i << 16);  // both counts stay below 2^16: one register through the DPP sums
+                    both += dpp_xor1(both);
+                    both += dpp_xor2(both);
+                    if (PARTS >= 8) both += dpp_half_mirror(both);
+                    if (PARTS >= 16) both += dpp_row_mirror(both);
+                    cnt = both & 0xffffu;
+                    cnt_i = both >> 16;
                     if (c < nc && part == 0) {
                         const uint32_t kmax = sh.cand_kmax;
                         sh.c.raw[cnt] = ki;
@@ -428,7 +438,10 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                         by_index_w(sh)[cnt_i] = 0;
                         by_index_idx(sh)[cnt_i] = ii;
                     }
-                }
+                };
+                if (nc <= 64u) rank_candidates(std::integral_constant<uint32_t, 16>{});
+                else if (nc <= 128u) rank_candidates(std::integral_constant<uint32_t, 8>{});
+                else rank_candidates(std::integral_constant<uint32_t, 4>{});
                 __syncthreads();
                 KA_STAMP(5);   // candidates sorted
                 if (tid < kWave) {  // one wavefront finishes the row; the others are done
