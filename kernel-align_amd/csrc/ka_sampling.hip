@@ -18,6 +18,8 @@
 // (ka_sampling_topk.h), and for 16-bit dtypes the no-filter and dense-histogram paths (ka_sampling_dense.h).
 // For aligned fp32 rows outside the candidate list a variant of the kernel replaces the last pass by a draw
 // over shares of the row (ka_sampling_draw.h).
+#include <mutex>
+
 #include "ka_sampling_common.h"
 #include "ka_sampling_dense.h"
 #include "ka_sampling_topk.h"
@@ -368,9 +370,22 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
     }
     if constexpr (T::kBytes == 2) {
       if (dense) {
-        const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(sample_rows<T, true>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, int(DENSE_LDS_BYTES));
-        if (rc != hipSuccess) return check_hip(rc, "sample: reserving LDS for the dense-histogram path");
+        // the attribute belongs to the device: set once per device and dtype, not per call
+        static std::mutex attr_mutex;
+        static bool attr_set[64] = {};
+        int device = 0;
+        hipError_t rc = hipGetDevice(&device);
+        if (rc != hipSuccess) return check_hip(rc, "sample: hipGetDevice");
+        if (device < 0 || device >= 64) return fail(KA_ERR_UNSUPPORTED, "sample: device index %d", device);
+        {
+            std::lock_guard<std::mutex> lock(attr_mutex);
+            if (!attr_set[device]) {
+                rc = hipFuncSetAttribute(reinterpret_cast<const void *>(sample_rows<T, true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(DENSE_LDS_BYTES));
+                if (rc != hipSuccess) return check_hip(rc, "sample: reserving LDS for the dense-histogram path");
+                attr_set[device] = true;
+            }
+        }
         hipLaunchKernelGGL((sample_rows<T, true>), dim3(unsigned(batch)), dim3(S_THREADS), DENSE_LDS_BYTES, stream, lp,
                            int(vocab), row_stride, prm, aligned ? 1 : 0, path_bits & 2);
         return check_hip(hipGetLastError(), "sample launch");
