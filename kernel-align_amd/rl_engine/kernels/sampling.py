@@ -39,6 +39,34 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} must live on the GPU: rl_engine has no CPU path (got {t.device})")
 
 
+class _NoGuard:
+    """Stands in for torch.cuda.device(...) when the tensor's device is the current one already."""
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device(device):
+    """A context manager that makes `device` current for the launch.  Entering torch.cuda.device() and asking
+    torch.cuda.current_stream() cost more host time than a small kernel runs, so the common case (the tensor lives
+    on the current device) takes neither."""
+    index = device.index
+    if index is None or index == torch._C._cuda_getDevice():
+        return _NO_GUARD
+    return torch.cuda.device(index)
+
+
+def _raw_stream() -> int:
+    """Handle of the current HIP stream of the current device (what torch.cuda.current_stream().cuda_stream returns)."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+
+
 def _chunk_rows(chunk_tokens) -> int:
     """Rows per launch of a chunked operator; anything below one row would make the launch loop empty."""
     chunk = DEFAULT_CHUNK_TOKENS if chunk_tokens is None else int(chunk_tokens)
@@ -114,8 +142,8 @@ class SamplerBackend(nn.Module):
         chunk = _chunk_rows(chunk_tokens)
         row_stride = rows.stride(0) if n_rows > 1 else vocab
         esize = rows.element_size()
-        with torch.cuda.device(logits.device):
-            stream = torch.cuda.current_stream().cuda_stream
+        with _on_device(logits.device):
+            stream = _raw_stream()
             base, ids_base, out_base = rows.data_ptr(), ids.data_ptr(), out.data_ptr()
             for start in range(0, n_rows, chunk):
                 n = min(chunk, n_rows - start)
@@ -146,8 +174,8 @@ class SamplerBackend(nn.Module):
         ent = torch.empty(n_rows, dtype=torch.float32, device=logits.device)
         row_stride = rows.stride(0) if n_rows > 1 else vocab
         esize = rows.element_size()
-        with torch.cuda.device(logits.device):
-            stream = torch.cuda.current_stream().cuda_stream
+        with _on_device(logits.device):
+            stream = _raw_stream()
             for start in range(0, n_rows, chunk):
                 n = min(chunk, n_rows - start)
                 status = fn(rows.data_ptr() + start * row_stride * esize, n, vocab, row_stride,
@@ -188,8 +216,8 @@ class SamplerBackend(nn.Module):
         esize = rows.element_size()
         chunk = _chunk_rows(chunk_tokens)
         fn = getattr(self._lib, fn_name)
-        with torch.cuda.device(logits.device):
-            stream = torch.cuda.current_stream().cuda_stream
+        with _on_device(logits.device):
+            stream = _raw_stream()
             for start in range(0, n_rows, chunk):
                 n = min(chunk, n_rows - start)
                 status = fn(rows.data_ptr() + start * row_stride * esize, n, vocab, row_stride,
@@ -232,12 +260,12 @@ class SamplerBackend(nn.Module):
         loss = torch.empty(n, dtype=torch.float32, device=new.device)
         kl = torch.empty_like(loss)
         dlogp = torch.empty_like(loss)
-        with torch.cuda.device(new.device):
+        with _on_device(new.device):
             status = self._lib.ka_grpo_token_terms(
                 new.data_ptr(), old.data_ptr() if old is not None else None,
                 ref.data_ptr() if ref is not None else None, adv.data_ptr(), n, float(clip_low), float(clip_high),
                 float(beta), loss.data_ptr(), kl.data_ptr(), dlogp.data_ptr(),
-                torch.cuda.current_stream().cuda_stream)
+                _raw_stream())
         _hip.check(status, "ka_grpo_token_terms")
         return loss.view(shape), kl.view(shape), dlogp.view(shape)
 
@@ -306,20 +334,25 @@ class SamplerBackend(nn.Module):
         ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
         row_stride = rows.stride(0) if batch > 1 else vocab
         extended = return_logprob or k_rows is not None or p_rows is not None or t_rows is not None or route_flags
-        with torch.cuda.device(dev), self._workspace(ws_bytes, dev) as ws_ptr:
-            stream = torch.cuda.current_stream().cuda_stream
+        def launch(ws_ptr):
+            stream = _raw_stream()
             if extended:
-                fn_name = "ka_sample_ex"
                 ptr = lambda x: None if x is None else x.data_ptr()  # noqa: E731
-                status = self._lib.ka_sample_ex(
+                return "ka_sample_ex", self._lib.ka_sample_ex(
                     _DTYPE_CODE[logits.dtype], rows.data_ptr(), batch, vocab, row_stride, t, ptr(t_rows), k,
                     ptr(k_rows), p, ptr(p_rows), uniforms.data_ptr(), out.data_ptr(), ptr(logprob),
                     int(route_flags), ws_ptr, ws_bytes, stream)
+            name = _SAMPLE_FN[logits.dtype]
+            return name, getattr(self._lib, name)(
+                rows.data_ptr(), batch, vocab, row_stride, t, k, p, uniforms.data_ptr(),
+                out.data_ptr(), ws_ptr, ws_bytes, stream)
+
+        with _on_device(dev):
+            if ws_bytes == 0:  # the kernels keep their state in LDS and registers: no lease, no event
+                fn_name, status = launch(None)
             else:
-                fn_name = _SAMPLE_FN[logits.dtype]
-                status = getattr(self._lib, fn_name)(
-                    rows.data_ptr(), batch, vocab, row_stride, t, k, p, uniforms.data_ptr(),
-                    out.data_ptr(), ws_ptr, ws_bytes, stream)
+                with self._workspace(ws_bytes, dev) as ws_ptr:
+                    fn_name, status = launch(ws_ptr)
         _hip.check(status, fn_name)
         return (out, logprob) if return_logprob else out
 
@@ -362,8 +395,8 @@ class SamplerBackend(nn.Module):
         if rows_per_call < 1:
             raise PoolExhausted(f"the {self.pool.capacity} B pool cannot hold the lm_head partials of one "
                                 f"256-token tile ({256 * per_row} B)")
-        with torch.cuda.device(hidden.device):
-            stream = torch.cuda.current_stream().cuda_stream
+        with _on_device(hidden.device):
+            stream = _raw_stream()
             for start in range(0, n_rows, rows_per_call):
                 n = min(rows_per_call, n_rows - start)
                 ws_bytes = self._lib.ka_lmhead_workspace_bytes(n, hdim, vocab)
