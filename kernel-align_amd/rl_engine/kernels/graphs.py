@@ -1,0 +1,61 @@
+"""A decode step of a rollout captured in a HIP graph.
+
+A decode step is two operator calls (sample, then the drawn token's log-probability under the unfiltered
+distribution, which a GRPO ratio is built from).  Both operators only launch kernels on the current stream - no
+allocation inside the library, no memset, no host synchronisation - so the step can be recorded once and replayed,
+alone or as part of a larger capture (the model's forward pass in front of it).
+Measured on an MI355X with ROCm 7.2 (bf16, 128,256 entries, top_k 50 + top_p 0.9): replaying this two-kernel graph on
+its own costs 26 us per step at 64 rows against 22 us for the two eager calls (a graph launch costs more here than
+two kernel launches), so on its own it buys nothing; its use is inside a capture that holds more work, and the test of
+it shows that the operators can be captured at all.
+
+    step = GraphedDecodeStep(sampler, batch=64, vocab=128256, top_k=50, top_p=0.9, temperature=0.7)
+    step.logits.copy_(next_logits)          # or let the model write into step.logits
+    step.uniforms.copy_(torch.rand(64))
+    ids, logp = step()                      # tensors owned by the step, overwritten by the next replay
+
+The reference has no counterpart (its operators are plain eager calls, rl_engine/kernels/sampling.py:39-112).
+"""
+from __future__ import annotations
+
+import torch
+
+
+class GraphedDecodeStep:
+    def __init__(self, sampler, batch: int, vocab: int, dtype=torch.bfloat16, top_k=None, top_p=None,
+                 temperature: float = 1.0, device="cuda", with_logprob: bool = True):
+        if batch < 1 or vocab < 1:
+            raise ValueError("batch and vocab must be positive")
+        self.sampler = sampler
+        dev = torch.device(device)
+        self.logits = torch.zeros(batch, vocab, dtype=dtype, device=dev)     # inputs: filled by the caller
+        self.uniforms = torch.zeros(batch, dtype=torch.float32, device=dev)
+        self.ids = None                                                       # outputs: owned by the graph
+        self.logp = None
+        self._kw = dict(top_k=top_k, top_p=top_p, temperature=temperature)
+        self._with_logprob = with_logprob
+        # torch wants a few eager runs on a side stream before it records (lazy initialisation must not be captured)
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                self._run()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.ids, self.logp = self._run()
+
+    def _run(self):
+        ids = self.sampler.sample(self.logits, uniforms=self.uniforms, **self._kw)
+        logp = self.sampler.compute_logp(self.logits, ids) if self._with_logprob else None
+        return ids, logp
+
+    def __call__(self, logits=None, uniforms=None):
+        """Replay the step.  `logits` / `uniforms`, if given, are copied into the step's input buffers first."""
+        if logits is not None:
+            self.logits.copy_(logits)
+        if uniforms is not None:
+            self.uniforms.copy_(uniforms)
+        self.graph.replay()
+        return self.ids, self.logp

@@ -95,3 +95,33 @@ def test_generate_loop_matches_stepwise_oracle():
         assert (logp[:, s].cpu() - lp).abs().max().item() <= 1e-4
         cur = tok
     assert done.any()
+
+
+def test_decode_step_replayed_from_a_hip_graph(sampler):
+    """GraphedDecodeStep records sample + compute_logp once and replays them: every replay - with the program's own
+    eager work and synchronisations between them - must give the eager operators' results bit for bit, and those
+    of the CPU oracles."""
+    from oracle import exact, logprob_ref
+    from rl_engine.kernels.graphs import GraphedDecodeStep
+
+    batch, vocab = 24, 32000
+    step = GraphedDecodeStep(sampler, batch, vocab, top_k=50, top_p=0.9, temperature=0.7)
+    g = torch.Generator().manual_seed(71)
+    for it in range(4):
+        logits = (torch.randn(batch, vocab, generator=g) * 3).bfloat16()
+        u = torch.rand(batch, generator=g)
+        if it % 2 == 0:
+            ids, logp = step(logits.cuda(), u.cuda())
+        else:                                          # the caller writes the inputs itself
+            step.logits.copy_(logits.cuda())
+            step.uniforms.copy_(u.cuda())
+            ids, logp = step()
+        got_ids, got_logp = ids.clone(), logp.clone()
+        torch.cuda.synchronize()
+        eager_ids = sampler.sample(logits.cuda(), top_k=50, top_p=0.9, temperature=0.7, uniforms=u.cuda())
+        eager_logp = sampler.compute_logp(logits.cuda(), eager_ids)
+        junk = torch.randn(1 << 20, device="cuda").sum().item()          # eager work and a sync between replays
+        assert junk == junk
+        assert torch.equal(got_ids, eager_ids) and torch.equal(got_logp, eager_logp)
+        assert torch.equal(got_ids.cpu(), exact.sample(logits, 0.7, 50, 0.9, u))
+        assert (got_logp.cpu() - logprob_ref.logprob_ref(logits, got_ids.cpu())).abs().max().item() <= 1e-4
