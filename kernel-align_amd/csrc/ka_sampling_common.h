@@ -175,18 +175,46 @@ struct alignas(16) Shared {
     DenseScalars ds;  // scalars of the resident no-filter path
 };
 
+// Inclusive prefix sum of one 64-bit value per lane over the wavefront, by DPP row shifts and row broadcasts.
+// One step: lanes outside ROW_MASK, and lanes whose source lies outside the row, add 0.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint64_t scan_step_u64(uint64_t v) {
+    const uint32_t lo = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v)), CTRL, ROW_MASK, 0xf, true));
+    const uint32_t hi = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v >> 32)), CTRL, ROW_MASK, 0xf, true));
+    return v + ((uint64_t(hi) << 32) | lo);
+}
+__device__ __forceinline__ uint64_t wave_incl_scan_u64(uint64_t v) {
+    v = scan_step_u64<0x111, 0xf>(v);  // row_shr:1
+    v = scan_step_u64<0x112, 0xf>(v);  // row_shr:2
+    v = scan_step_u64<0x114, 0xf>(v);  // row_shr:4
+    v = scan_step_u64<0x118, 0xf>(v);  // row_shr:8
+    v = scan_step_u64<0x142, 0xa>(v);  // row_bcast:15 -> rows 1 and 3
+    v = scan_step_u64<0x143, 0xc>(v);  // row_bcast:31 -> rows 2 and 3
+    return v;
+}
+
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint32_t scan_step_u32(uint32_t v) {
+    return v + uint32_t(__builtin_amdgcn_update_dpp(0, int(v), CTRL, ROW_MASK, 0xf, true));
+}
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v) {
+    v = scan_step_u32<0x111, 0xf>(v);
+    v = scan_step_u32<0x112, 0xf>(v);
+    v = scan_step_u32<0x114, 0xf>(v);
+    v = scan_step_u32<0x118, 0xf>(v);
+    v = scan_step_u32<0x142, 0xa>(v);
+    v = scan_step_u32<0x143, 0xc>(v);
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) { return wave_incl_scan_u32(v); }
+__device__ __forceinline__ uint64_t wave_incl_scan(uint64_t v) { return wave_incl_scan_u64(v); }
+
 template <typename V> __device__ __forceinline__ V shfl_up_v(V v, int off) { return __shfl_up(v, off, kWave); }
 
-// Exclusive prefix sum over the block in thread order; *total = block sum.  Contains barriers.
+// Exclusive prefix sum over the block in thread order; *total = block sum.  Contains barriers; every thread of the
+// block must call it (the wavefront-level part moves data by DPP, which needs all 64 lanes active).
 template <typename V>
 __device__ __forceinline__ V block_excl_scan(V v, V *wave_buf, V *total) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    V inc = v;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const V t = shfl_up_v(inc, off);
-        if (lane >= off) inc += t;
-    }
+    const V inc = wave_incl_scan(v);
     __syncthreads();  // wave_buf may still be read from a previous call
     if (lane == kWave - 1) wave_buf[wave] = inc;
     __syncthreads();

@@ -24,13 +24,14 @@ namespace {
 // ---------------------------------------------------------------------------
 
 // ---------------------------------------------------------------------------
-// Pieces of the short route (top_k <= SHORT_TOPK): after the read of the row, five block-wide barriers and a tail on
+// Pieces of the short route (top_k <= SHORT_TOPK): after the read of the row, a handful of block-wide barriers and a tail on
 // one wavefront instead of radix descents and block-wide scans.
 // ---------------------------------------------------------------------------
-constexpr int SHORT_TOPK = 64;    // largest top_k the short route serves
-constexpr int SHORT_GROUPS = 128; // the 1024 lane maxima are pooled into this many group maxima (8 lanes each)
-constexpr int SHORT_VECS = 128;   // candidate vectors the short route takes (128 * 8 elements = one per thread)
-constexpr int SHORT_CAND = 256;   // candidates its tail takes (four per lane of one wavefront)
+constexpr int SHORT_TOPK = 256;      // largest top_k the short route serves
+constexpr int SHORT_POOL_TOPK = 64;  // up to here the bound comes from pooled group maxima, above from a radix descent
+constexpr int SHORT_GROUPS = 128;    // the 1024 lane maxima are pooled into this many group maxima (8 lanes each)
+constexpr int SHORT_VECS = 512;      // candidate vectors the short route takes (16 bytes each in LDS)
+constexpr int SHORT_CAND = 512;      // candidates its tail takes (eight per lane of one wavefront)
 
 // Cross-lane moves inside a row of sixteen lanes (DPP: no LDS traffic): lane ^ 1, lane ^ 2, 7 - lane inside each
 // half row, and 15 - lane.  Applied in this order, a sum (or maximum) over 2, 4, 8, 16 neighbouring lanes builds up.
@@ -38,23 +39,6 @@ __device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) { return uint32_t(__bui
 __device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)); }
 __device__ __forceinline__ uint32_t dpp_row_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)); }
 __device__ __forceinline__ uint32_t dpp_half_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)); }
-
-// Inclusive prefix sum of one 64-bit value per lane over the wavefront, by DPP row shifts and row broadcasts.
-// One step: lanes outside ROW_MASK, and lanes whose source lies outside the row, add 0.
-template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint64_t scan_step_u64(uint64_t v) {
-    const uint32_t lo = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v)), CTRL, ROW_MASK, 0xf, true));
-    const uint32_t hi = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v >> 32)), CTRL, ROW_MASK, 0xf, true));
-    return v + ((uint64_t(hi) << 32) | lo);
-}
-__device__ __forceinline__ uint64_t wave_incl_scan_u64(uint64_t v) {
-    v = scan_step_u64<0x111, 0xf>(v);  // row_shr:1
-    v = scan_step_u64<0x112, 0xf>(v);  // row_shr:2
-    v = scan_step_u64<0x114, 0xf>(v);  // row_shr:4
-    v = scan_step_u64<0x118, 0xf>(v);  // row_shr:8
-    v = scan_step_u64<0x142, 0xa>(v);  // row_bcast:15 -> rows 1 and 3
-    v = scan_step_u64<0x143, 0xc>(v);  // row_bcast:31 -> rows 2 and 3
-    return v;
-}
 
 // Minimum of one value per lane over the wavefront, in every lane (DPP row shifts and broadcasts, then lane 63).
 template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint32_t min_step_u32(uint32_t v) {
@@ -77,7 +61,8 @@ __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
 //   by_index_w(sh)[q], by_index_idx(sh)[q]  mass (0 until the tail files the kept ones) and index of the candidate
 //                                           that is q-th in ascending index order.
 __device__ __forceinline__ uint64_t *by_index_w(Shared &sh) { return sh.c.w + SHORT_CAND; }
-__device__ __forceinline__ uint32_t *by_index_idx(Shared &sh) { return reinterpret_cast<uint32_t *>(sh.c.w + 2 * SHORT_CAND); }
+__device__ __forceinline__ uint32_t *by_index_idx(Shared &sh) { return sh.c.sidx + SHORT_CAND; }
+static_assert(2 * SHORT_CAND <= CAND_CAP && SHORT_VECS * 16 <= CAND_CAP * 8, "the short route's lists live in the candidate area");
 
 // The tail of the short route on one wavefront, after the block has ranked the nc <= SHORT_CAND candidates both ways.
 // Position p of the key order is handled by slot p / 64 of lane p % 64; na <= 64 * SLOTS positions hold the top-k
@@ -285,8 +270,30 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         }
         return guard < 64;
     };
+    // the top_k-th largest of the 1024 lane maxima, by the same MSB-first descent over count histograms as the radix path
+    auto radix_bound = [&]() -> uint32_t {
+        const uint32_t lmax = masked_key<T>(lmaxf);
+        uint32_t rank = uint32_t(top_k), prefix = 0;
+        for (int level = 0; level < Round<T>::kLevels; ++level) {
+            const int shift = level_shift<T>(level), bits = level_bits<T>(level);
+            const uint32_t nb = 1u << bits;
+            __syncthreads();
+            for (int b = tid; b < int(nb); b += S_THREADS) sh.h.cnt[b] = 0;
+            __syncthreads();
+            if (level == 0 || (lmax >> level_shift<T>(level - 1)) == prefix)
+                atomicAdd(&sh.h.cnt[(lmax >> shift) & (nb - 1)], 1u);
+            __syncthreads();
+            uint32_t above, count;
+            const uint32_t digit = select_count_bin(sh, nb, rank, &above, &count);
+            prefix = (prefix << bits) | digit;
+            rank -= above;
+        }
+        return prefix << level_shift<T>(Round<T>::kLevels - 1);
+    };
     bool have_candidates = false;  // the short route has filled the candidate list but leaves the tail to the block
     if (short_route) {
+        uint32_t bound;
+        if (top_k <= SHORT_POOL_TOPK) {
         // S1. The lane maxima are pooled into 128 group maxima (eight neighbouring lanes each); the top_k-th largest
         //     group maximum is a lower bound of the top_k-th largest element (each group maximum is a different
         //     element), and with top_k well below 128 nearly as tight as the top_k-th largest lane maximum.
@@ -321,8 +328,14 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
             if (part == 0 && cnt == uint32_t(top_k - 1)) sh.max_key = __float_as_uint(x);
         }
         __syncthreads();
+        bound = masked_key<T>(__uint_as_float(sh.max_key));
+        } else {
+            // 64 < top_k <= 256: the exact top_k-th largest lane maximum (128 pooled maxima would be too few)
+            bound = radix_bound();
+            if (tid == 0) { sh.n_cand = 0; sh.n_vec = 0; sh.hit = -1; sh.cand_kmax = 0; }
+            __syncthreads();
+        }
         KA_STAMP(2);   // bound known
-        uint32_t bound = masked_key<T>(__uint_as_float(sh.max_key));
         if (!widen_bound(bound)) return false;
         KA_STAMP(3);   // bound widened
         const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
@@ -384,8 +397,8 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         const uint32_t nv = sh.n_vec;
         if (nv <= uint32_t(SHORT_VECS)) {
             // S4. One thread per element of the listed vectors: those at or above the bound join the candidate list.
-            if (tid < int(nv) * EPV) {
-                const int vslot = tid / EPV, e = tid % EPV;
+            for (int i = tid; i < int(nv) * EPV; i += S_THREADS) {
+                const int vslot = i / EPV, e = i % EPV;
                 const typename T::raw_t raw = reinterpret_cast<const typename T::raw_t *>(cvec + vslot)[e];
                 add_element(int(cvidx[vslot]) * EPV + e, raw);
             }
@@ -398,7 +411,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                 //     alone, and file it under both ranks together with its integer mass (see by_index_w above; none
                 //     of the arrays written here is read in this step).
                 uint32_t *const rank_by_index = sh.c.raw + SHORT_CAND;  // [key rank] -> position in index order
-                // PARTS threads share a candidate (16 for up to 64 candidates, 8 up to 128, 4 up to 256: all 1024
+                // PARTS threads share a candidate (16 for up to 64 candidates, 8 up to 128, 4 up to 256, 2 up to 512: all 1024
                 // threads take part), each over every PARTS-th group of four entries; the counts are summed inside the
                 // PARTS neighbouring lanes by DPP.
                 auto rank_candidates = [&](auto parts_c) {
@@ -424,7 +437,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                     }
                     uint32_t both = cnt | (cnt_i << 16);  // both counts stay below 2^16: one register through the DPP sums
                     both += dpp_xor1(both);
-                    both += dpp_xor2(both);
+                    if (PARTS >= 4) both += dpp_xor2(both);
                     if (PARTS >= 8) both += dpp_half_mirror(both);
                     if (PARTS >= 16) both += dpp_row_mirror(both);
                     cnt = both & 0xffffu;
@@ -441,7 +454,8 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                 };
                 if (nc <= 64u) rank_candidates(std::integral_constant<uint32_t, 16>{});
                 else if (nc <= 128u) rank_candidates(std::integral_constant<uint32_t, 8>{});
-                else rank_candidates(std::integral_constant<uint32_t, 4>{});
+                else if (nc <= 256u) rank_candidates(std::integral_constant<uint32_t, 4>{});
+                else rank_candidates(std::integral_constant<uint32_t, 2>{});
                 __syncthreads();
                 KA_STAMP(5);   // candidates sorted
                 if (tid < kWave) {  // one wavefront finishes the row; the others are done
@@ -455,37 +469,18 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                     }
                     if (na <= uint32_t(kWave)) short_tail<T, 1>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
                     else if (na <= uint32_t(2 * kWave)) short_tail<T, 2>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
-                    else short_tail<T, 4>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
+                    else if (na <= uint32_t(4 * kWave)) short_tail<T, 4>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
+                    else short_tail<T, 8>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
                     KA_STAMP(9);
                 }
                 return true;
             }
-            have_candidates = true;  // more than 256 candidates (a large tie group): the block-wide tail ranks them
+            have_candidates = true;  // more than 512 candidates (a large tie group): the block-wide tail ranks them
         }
         __syncthreads();  // too many candidate vectors: the block-wide route starts over with its exact bound
     }
     if (!have_candidates) {
-    uint32_t bound = 0;
-    const uint32_t lmax = masked_key<T>(lmaxf);
-    // the top_k-th largest of the 1024 lane maxima, by the same MSB-first descent over count histograms
-    {
-        uint32_t rank = uint32_t(top_k), prefix = 0;
-        for (int level = 0; level < Round<T>::kLevels; ++level) {
-            const int shift = level_shift<T>(level), bits = level_bits<T>(level);
-            const uint32_t nb = 1u << bits;
-            __syncthreads();
-            for (int b = tid; b < int(nb); b += S_THREADS) sh.h.cnt[b] = 0;
-            __syncthreads();
-            if (level == 0 || (lmax >> level_shift<T>(level - 1)) == prefix)
-                atomicAdd(&sh.h.cnt[(lmax >> shift) & (nb - 1)], 1u);
-            __syncthreads();
-            uint32_t above, count;
-            const uint32_t digit = select_count_bin(sh, nb, rank, &above, &count);
-            prefix = (prefix << bits) | digit;
-            rank -= above;
-        }
-        bound = prefix << level_shift<T>(Round<T>::kLevels - 1);
-    }
+    uint32_t bound = radix_bound();
     if (tid == 0) { sh.n_cand = 0; sh.hit = -1; }
     __syncthreads();
     KA_STAMP(2);   // bound known

@@ -228,8 +228,9 @@ def test_fast_and_radix_paths_are_the_same_function(sampler):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_wavefront_route_of_small_top_k(sampler, dtype):
-    """top_k <= 64 bounds the candidates from per-wavefront sorted lane maxima and finishes on one wavefront with
-    1, 2 or 4 candidates per lane; beyond 256 candidates, or with top_k = 65, the block-wide tail takes over.
+    """top_k <= 256 takes the short route (bound from pooled group maxima up to 64, from a radix descent above; tail on
+    one wavefront with 1 to 8 candidates per lane); beyond 512 candidates, or with top_k = 257, the block-wide route
+    takes over.
     Rows are built to hit each of those sizes: smooth rows (few candidates), coarse grids (tie groups of tens to
     hundreds of entries at the k-th value), a cut inside a tie group, the largest values packed into the share of
     one lane / one wavefront (loose bounds), and all three routes must give the oracle's ids and log-probabilities."""
@@ -246,7 +247,7 @@ def test_wavefront_route_of_small_top_k(sampler, dtype):
     for rows, temps in ((smooth, (0.7, 1.0)), (coarse, (1.0, 0.5)), (coarser, (1.0,)), (packed, (0.7,)), (flat, (1.0,))):
         logits = rows.to(dtype)
         u = torch.rand(logits.shape[0], generator=g)
-        for k in (1, 2, 17, 50, 63, 64, 65):
+        for k in (1, 2, 17, 50, 63, 64, 65, 130, 200, 256, 257):
             for p in (None, 0.9, 0.3):
                 for temp in temps:
                     want, want_lp = exact.sample_rows(logits, temp, k, p, u)
