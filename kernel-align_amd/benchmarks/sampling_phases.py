@@ -1,5 +1,6 @@
 """Where the cycles of one sampling call go: builds the sampling kernels with -DKA_SAMPLE_STAMPS (workgroup 0 then
-writes the shader clock at named points of the top-k route) and prints the phases for B in {1, 64, 256}.
+writes the shader clock at named points of the top-k route and of the dense-histogram route) and prints the phases for
+B in {1, 64, 256} (top-k + top-p) and B in {64, 256} (top-p alone, at T = 0.7 and T = 1).
 
     python kernel-align_amd/benchmarks/sampling_phases.py [--top-k 50] [--top-p 0.9] [--temperature 0.7]
 
@@ -79,6 +80,24 @@ def main() -> int:
                     prev = st[i]
             print(f"B={batch:4d} {label:16s} {prev - st[0]:6d} cycles (wavefront 0; last wavefront has read its share at "
                   f"{last_read}): " + " | ".join(parts), flush=True)
+    # the dense-histogram route (top-p without top-k): its own stamp names
+    dense_names = {1: "histogram pass", 2: "occupied keys compacted", 3: "masses of the occupied keys",
+                   4: "filters + mass table", 11: "survivors listed", 12: "drawn"}
+    for batch in (64, 256):
+        logits, u = cfg5_sampling(batch, device="cuda")
+        for temp in (0.7, 1.0):
+            for _ in range(3):
+                sampler.sample(logits, top_p=args.top_p, temperature=temp, uniforms=u)
+            torch.cuda.synchronize()
+            lib.ka_debug_read_stamps(buf, 288)
+            st = list(buf)
+            prev, parts = st[0], []
+            for i in (1, 2, 3, 4, 11, 12):
+                if st[i] > prev:
+                    parts.append(f"{dense_names[i]} +{st[i] - prev}")
+                    prev = st[i]
+            tail = "" if st[12] > st[4] else " | (more than 2048 survivors: streaming draw, not stamped)"
+            print(f"B={batch:4d} top_p={args.top_p} T={temp}: stamped {prev - st[0]:6d} cycles: " + " | ".join(parts) + tail, flush=True)
     return 0
 
 

@@ -3,6 +3,8 @@
 #ifndef KA_SAMPLING_COMMON_H
 #define KA_SAMPLING_COMMON_H
 
+#include <type_traits>
+
 #include "ka_common.h"
 
 namespace ka {
@@ -153,6 +155,8 @@ struct DenseScalars {
     uint32_t seg_ties[S_WAVES + 1];  // ... and its number of tie-group entries
     uint64_t z_topk, before_cut, w_cut, pick_w;
     uint32_t i_topk, n_cut, kcut16, i_last, tie_hi, tie_lo, fail, n_inf;
+    uint32_t n_ge, surv_overflow;    // dense path: entries at or above the lowest surviving key; a wavefront's survivor list overflowed
+    uint32_t seg_cnt[S_WAVES];       // ... survivors listed by each wavefront
     int best_i;
     int64_t hit;
 };
@@ -174,6 +178,13 @@ struct alignas(16) Shared {
     uint64_t pick_z;
     DenseScalars ds;  // scalars of the resident no-filter path
 };
+
+// Cross-lane moves inside a row of sixteen lanes (DPP: no LDS traffic): lane ^ 1, lane ^ 2, 7 - lane inside each
+// half row, and 15 - lane.  Applied in this order, a sum (or maximum) over 2, 4, 8, 16 neighbouring lanes builds up.
+__device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)); }
+__device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)); }
+__device__ __forceinline__ uint32_t dpp_row_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)); }
+__device__ __forceinline__ uint32_t dpp_half_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)); }
 
 // Inclusive prefix sum of one 64-bit value per lane over the wavefront, by DPP row shifts and row broadcasts.
 // One step: lanes outside ROW_MASK, and lanes whose source lies outside the row, add 0.

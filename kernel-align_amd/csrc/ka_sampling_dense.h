@@ -34,6 +34,9 @@ constexpr int D_WORDS = 32768;              // 65,536 16-bit counters
 constexpr int D_LIST_CAP = 7168;            // occupied keys the list can hold (4 B each)
 constexpr int D_TABLE_CAP = D_LIST_CAP / 2; // keys spanned by the survivors (8 B each, same LDS region)
 constexpr int D_PER_THREAD = D_LIST_CAP / S_THREADS;  // list entries per thread
+constexpr int D_SURV_SEG = 512;             // survivors per wavefront the list-based draw of the filtered modes takes (12 B each)
+constexpr int D_SURV_DEFER = 2048;          // ... and in all (more survivors: the streaming draw is faster)
+static_assert(size_t(S_WAVES + 1) * D_SURV_SEG * 12 <= size_t(D_WORDS) * 4, "the survivor lists live in the histogram's memory");
 
 constexpr size_t DENSE_LDS_BYTES = size_t(D_WORDS) * 4 + size_t(D_LIST_CAP) * 4 + sizeof(DenseScalars);
 
@@ -476,6 +479,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     __syncthreads();  // ds.n_inf is zero
     if ((tid & (kWave - 1)) == 0 && my_inf != 0) atomicAdd(&ds.n_inf, my_inf);
     const uint32_t kmax = block_max_u32_buf(lmax, ds.wave_u32);  // largest raw key; the barriers also publish the histogram
+    KA_STAMP(1);   // histogram pass
     if (kmax == kNegInfKey) return false;  // nothing above -inf: the draw is uniform over the row (radix path)
     const uint32_t n_inf = ds.n_inf;
 
@@ -516,6 +520,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     }
     __syncthreads();
 
+    KA_STAMP(2);   // occupied keys compacted
     // ---- 3. scaled key and mass, once per occupied key: lane t takes the entries [t * D_PER_THREAD, ...) -------
     // Several raw keys may scale to one value; such a run of entries is one tie group of the operator.
     uint16_t *const skl = reinterpret_cast<uint16_t *>(hist);  // scaled key of every list entry (the counts are spent)
@@ -552,6 +557,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         ds.fail = 0;
     }
     __syncthreads();  // skl[] complete
+    KA_STAMP(3);   // masses of the occupied keys
     // last entry of the run (equal scaled keys) that contains entry i; a run longer than 64 entries (a huge
     // temperature folds many values together) is left to the radix path
     auto run_end = [&](uint32_t i) -> uint32_t {
@@ -674,10 +680,18 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     if (ds.fail) return false;
     // ---- 6. masses of the surviving raw keys into a table indexed by key - lowest surviving key ---------------
     if (tid == i_last / D_PER_THREAD) {
+        uint32_t c_run = c_before;
 #pragma unroll
-        for (int e = 0; e < D_PER_THREAD; ++e)
-            if (uint32_t(tid) * D_PER_THREAD + e == i_last) ds.kcut16 = ent[e] >> 16;
+        for (int e = 0; e < D_PER_THREAD; ++e) {
+            c_run += ent[e] & 0xffffu;
+            if (uint32_t(tid) * D_PER_THREAD + e == i_last) {
+                ds.kcut16 = ent[e] >> 16;
+                ds.n_ge = c_run;  // entries of the row at or above the lowest surviving key
+            }
+        }
     }
+    if (tid == 0) ds.surv_overflow = 0;
+    if (tid < S_WAVES) ds.seg_cnt[tid] = 0;
     __syncthreads();  // also: every lane is done reading the list
     kcut16 = ds.kcut16;
     span = kmax - kcut16 + 1;
@@ -693,11 +707,219 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
     (void)z_kept;  // equals the total the draw computes from the table
     first = track_ties ? tie_hi + 1 : kcut16;  // lowest raw key whose entries all survive
     }  // filters
+    auto is_tie = [&](uint32_t k) { return track_ties && k >= tie_lo && k <= tie_hi; };
+    KA_STAMP(4);   // filters and mass table
+    // ---- 7'. the survivors are few (a top-p nucleus of a peaked distribution, a top-k of a few thousand) and all
+    //          positive: list them and draw on the list instead of streaming the masses of the whole row -------------
+    // The row is read once more, but a vector only costs a packed signed maximum of its raw bits and a compare with the
+    // lowest surviving value (positive values order as their bit patterns).  The few vectors that hold a survivor are
+    // read again from L2, one per lane and turn, and their survivors go to a list per wavefront (the wavefront's share
+    // of the row is a contiguous sixteenth) with their masses.  The per-wavefront totals pick the share that holds
+    // floor(u * Z) exactly as in 7b; the block ranks that share's survivors by index, and one wavefront walks them with
+    // prefix sums.
+    if constexpr (!ALL_SURVIVE) {
+        const int lane = tid & (kWave - 1);
+        if (ds.n_ge <= uint32_t(D_SURV_DEFER) && kcut16 > 0x8000u && vpw <= 32 * kWave) {  // the same for the whole block
+            uint32_t *const s_idx = hist;                                                   // [S_WAVES][D_SURV_SEG], bit 31: tie-group entry
+            uint64_t *const s_w = reinterpret_cast<uint64_t *>(hist + S_WAVES * D_SURV_SEG);  // the histogram's memory is free by now
+            uint32_t *const o_idx = hist + 3 * S_WAVES * D_SURV_SEG;                         // the chosen share, in index order
+            uint64_t *const o_w = reinterpret_cast<uint64_t *>(o_idx + D_SURV_SEG);
+            // which of the lane's vectors hold a value at or above the cut (bit s: vector s * 64 + lane of the share)
+            const int cut_raw = int(kcut16 & 0x7fffu);
+            uint32_t hits = 0;
+#pragma unroll 1
+            for (int i0 = 0; i0 < n_here; i0 += 4 * kWave) {
+                uint4 q[4];
+#pragma unroll
+                for (int sq = 0; sq < 4; ++sq) {
+                    const int idx = i0 + sq * kWave + lane;
+                    q[sq] = idx < n_here ? vp[idx] : make_uint4(0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u);
+                }
+#pragma unroll
+                for (int sq = 0; sq < 4; ++sq) {
+                    i16x2 top = __builtin_elementwise_max(__builtin_bit_cast(i16x2, q[sq].x), __builtin_bit_cast(i16x2, q[sq].y));
+                    top = __builtin_elementwise_max(top, __builtin_elementwise_max(__builtin_bit_cast(i16x2, q[sq].z),
+                                                                                  __builtin_bit_cast(i16x2, q[sq].w)));
+                    const int best = top.x > top.y ? int(top.x) : int(top.y);  // a NaN pattern passes: sorted out below
+                    hits |= (best >= cut_raw ? 1u : 0u) << (i0 / kWave + sq);
+                }
+            }
+            uint64_t m_lane = 0;
+            uint32_t t_lane = 0;
+            bool overflow = false;
+            while (__any(hits != 0)) {
+                if (hits != 0) {
+                    const int sbit = __ffs(hits) - 1;
+                    hits &= hits - 1;
+                    const int idx = sbit * kWave + lane;
+                    uint32_t kk[4];
+                    vector_keys<T, false>(vp[idx], 1.0f, kk);
+                    uint32_t smask = 0;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) smask |= (key_at(kk, j) >= kcut16 ? 1u : 0u) << j;
+                    if (smask != 0) {
+                        const uint32_t cnt = uint32_t(__popc(smask));
+                        uint32_t pos = atomicAdd(&ds.seg_cnt[wave], cnt);
+                        if (pos + cnt <= uint32_t(D_SURV_SEG)) {
+                            pos += uint32_t(wave) * D_SURV_SEG;
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                if ((smask >> j) & 1u) {
+                                    const uint32_t key = key_at(kk, j);
+                                    const bool tie = is_tie(key);
+                                    const uint64_t wv = tie ? 0ull : table[key >= first ? key - kcut16 : span];
+                                    s_idx[pos] = uint32_t((v0 + idx) * 8 + j) | (tie ? 0x80000000u : 0u);
+                                    s_w[pos] = wv;
+                                    ++pos;
+                                    m_lane += wv;
+                                    t_lane += tie ? 1u : 0u;
+                                }
+                            }
+                        } else {
+                            overflow = true;
+                        }
+                    }
+                }
+            }
+            const uint64_t m = wave_sum_u64(m_lane);
+            const uint32_t t = wave_sum_u32(t_lane);
+            const bool tail_tie = has_tail && is_tie(tail_key);
+            uint64_t mt = (has_tail && !tail_tie && tail_key >= kcut16) ? table[tail_key >= first ? tail_key - kcut16 : span] : 0ull;
+            uint32_t tt = tail_tie ? 1u : 0u;
+            if (wave == 0) {
+                mt = wave_sum_u64(mt);
+                tt = wave_sum_u32(tt);
+            }
+            if (__any(overflow) && lane == 0) ds.surv_overflow = 1;
+            if (lane == 0) {
+                ds.seg_mass[wave] = m;
+                ds.seg_ties[wave] = t;
+                if (wave == 0) {
+                    ds.seg_mass[S_WAVES] = mt;
+                    ds.seg_ties[S_WAVES] = tt;
+                }
+            }
+            __syncthreads();
+            KA_STAMP(11);
+            if (!ds.surv_overflow) {  // (else a share holds more survivors than its list: the streaming draw below runs)
+                // the share (or the ragged tail) that holds floor(u * Z): as in 7b below
+                uint64_t z = 0;
+                {
+                    uint32_t seen = 0;
+#pragma unroll
+                    for (int g = 0; g <= S_WAVES; ++g) {
+                        const uint32_t tg = ds.seg_ties[g];
+                        const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
+                        z += ds.seg_mass[g] + uint64_t(tg < room ? tg : room) * w_tie;
+                        seen += tg;
+                    }
+                }
+                const uint64_t tau = floor_scale(u, z);
+                uint64_t acc = 0;
+                uint32_t ties_before = 0;
+                int seg = -1;
+                {
+                    uint32_t seen = 0;
+#pragma unroll
+                    for (int g = 0; g <= S_WAVES; ++g) {
+                        const uint32_t tg = ds.seg_ties[g];
+                        const uint32_t room = seen < r_cut ? r_cut - seen : 0u;
+                        const uint64_t mg = ds.seg_mass[g] + uint64_t(tg < room ? tg : room) * w_tie;
+                        if (seg < 0 && tau < acc + mg) { seg = g; ties_before = seen; }
+                        if (seg < 0) acc += mg;
+                        seen += tg;
+                    }
+                }
+                const uint32_t n = (seg >= 0 && seg < S_WAVES) ? ds.seg_cnt[seg] : 0u;
+                if (n > 0) {
+                    // the share's survivors were listed in no particular order: file them by index
+                    const uint32_t *const u_idx = s_idx + uint32_t(seg) * D_SURV_SEG;
+                    const uint64_t *const u_w = s_w + uint32_t(seg) * D_SURV_SEG;
+                    auto file_by_index = [&](auto parts_c) {
+                        constexpr uint32_t PARTS = decltype(parts_c)::value;
+                        const uint32_t c = uint32_t(tid) / PARTS, part = uint32_t(tid) % PARTS;
+                        uint32_t mine = 0, before = 0;
+                        if (c < n) {
+                            mine = u_idx[c];
+                            const uint4 *i4 = reinterpret_cast<const uint4 *>(u_idx);
+                            for (uint32_t g4 = part; g4 * 4 < n; g4 += PARTS) {
+                                const uint4 iq = i4[g4];
+                                const uint32_t ik[4] = {iq.x, iq.y, iq.z, iq.w};
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    before += (g4 * 4 + e < n && (ik[e] & 0x7fffffffu) < (mine & 0x7fffffffu)) ? 1u : 0u;
+                            }
+                        }
+                        before += dpp_xor1(before);
+                        if (PARTS >= 4) before += dpp_xor2(before);
+                        if (PARTS >= 8) before += dpp_half_mirror(before);
+                        if (PARTS >= 16) before += dpp_row_mirror(before);
+                        if (c < n && part == 0) {
+                            o_idx[before] = mine;
+                            o_w[before] = u_w[c];
+                        }
+                    };
+                    if (n <= 64u) file_by_index(std::integral_constant<uint32_t, 16>{});
+                    else if (n <= 128u) file_by_index(std::integral_constant<uint32_t, 8>{});
+                    else if (n <= 256u) file_by_index(std::integral_constant<uint32_t, 4>{});
+                    else file_by_index(std::integral_constant<uint32_t, 2>{});
+                    __syncthreads();
+                }
+                if (wave == 0) {
+                    int64_t hit = -1;
+                    uint64_t w_hit = 0;
+                    if (seg >= 0 && seg < S_WAVES) {
+                        uint64_t base = acc;
+                        uint32_t rank0 = ties_before;
+                        for (uint32_t q0 = 0; q0 < n; q0 += kWave) {  // wavefront-uniform
+                            const bool live = q0 + uint32_t(lane) < n;
+                            const uint32_t iw = live ? o_idx[q0 + lane] : 0u;
+                            const uint64_t wv = live ? o_w[q0 + lane] : 0ull;
+                            const bool tie = live && (iw >> 31) != 0;
+                            const uint64_t tmask = __ballot(tie);
+                            const uint32_t rank = rank0 + uint32_t(__popcll(tmask & ((uint64_t(1) << lane) - 1)));
+                            const uint64_t weff = tie ? (rank < r_cut ? w_tie : 0ull) : wv;
+                            const uint64_t inc = base + wave_incl_scan_u64(weff);
+                            const uint64_t above = __ballot(live && inc > tau);
+                            if (above != 0) {
+                                const int f = __ffsll((long long)above) - 1;
+                                hit = int64_t(uint32_t(__builtin_amdgcn_readlane(int(iw), f)) & 0x7fffffffu);
+                                w_hit = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(weff >> 32)), f))) << 32) |
+                                        uint32_t(__builtin_amdgcn_readlane(int(uint32_t(weff)), f));
+                                break;
+                            }
+                            base = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc >> 32)), kWave - 1))) << 32) |
+                                   uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc)), kWave - 1));
+                            rank0 += uint32_t(__popcll(tmask));
+                        }
+                    } else if (seg == S_WAVES) {  // the ragged tail: fewer than eight entries, one per lane
+                        const uint32_t rk = ties_before + wave_excl_scan<uint32_t>(tail_tie ? 1u : 0u);
+                        const uint64_t wt = has_tail ? (tail_tie ? (rk < r_cut ? w_tie : 0ull)
+                                                                 : (tail_key >= kcut16 ? table[tail_key >= first ? tail_key - kcut16 : span] : 0ull))
+                                                     : 0ull;
+                        const uint64_t before = acc + wave_excl_scan<uint64_t>(wt);
+                        const uint64_t above = __ballot(before <= tau && tau < before + wt);
+                        if (above != 0) {
+                            const int f = __ffsll((long long)above) - 1;
+                            hit = int64_t(nvec) * 8 + f;
+                            w_hit = (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(wt >> 32)), f))) << 32) |
+                                    uint32_t(__builtin_amdgcn_readlane(int(uint32_t(wt)), f));
+                        }
+                    }
+                    if (lane == 0) {
+                        *out_slot = hit;
+                        if (lp_slot != nullptr) *lp_slot = hit >= 0 ? log_ratio(w_hit, z) : __builtin_nanf("");
+                    }
+                    KA_STAMP(12);
+                }
+                return true;
+            }
+        }
+    }
     // ---- 7. draw over the survivors in index order ------------------------------------------------------------
     auto mass = [&](uint32_t k) -> uint64_t {
         return all_survive ? table[idx16[k]] : table[k >= first ? k - kcut16 : span];
     };
-    auto is_tie = [&](uint32_t k) { return track_ties && k >= tie_lo && k <= tie_hi; };
     // 7a. per wavefront: mass of the full survivors and number of tie-group entries of its share of the row
     {
         uint64_t m = 0;

@@ -2,8 +2,6 @@
 #ifndef KA_SAMPLING_TOPK_H
 #define KA_SAMPLING_TOPK_H
 
-#include <type_traits>
-
 #include "ka_sampling_common.h"
 
 namespace ka {
@@ -32,13 +30,6 @@ constexpr int SHORT_POOL_TOPK = 64;  // up to here the bound comes from pooled g
 constexpr int SHORT_GROUPS = 128;    // the 1024 lane maxima are pooled into this many group maxima (8 lanes each)
 constexpr int SHORT_VECS = 512;      // candidate vectors the short route takes (16 bytes each in LDS)
 constexpr int SHORT_CAND = 512;      // candidates its tail takes (eight per lane of one wavefront)
-
-// Cross-lane moves inside a row of sixteen lanes (DPP: no LDS traffic): lane ^ 1, lane ^ 2, 7 - lane inside each
-// half row, and 15 - lane.  Applied in this order, a sum (or maximum) over 2, 4, 8, 16 neighbouring lanes builds up.
-__device__ __forceinline__ uint32_t dpp_xor1(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)); }
-__device__ __forceinline__ uint32_t dpp_xor2(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)); }
-__device__ __forceinline__ uint32_t dpp_row_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)); }
-__device__ __forceinline__ uint32_t dpp_half_mirror(uint32_t v) { return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)); }
 
 // Minimum of one value per lane over the wavefront, in every lane (DPP row shifts and broadcasts, then lane 63).
 template <int CTRL, int ROW_MASK> __device__ __forceinline__ uint32_t min_step_u32(uint32_t v) {
