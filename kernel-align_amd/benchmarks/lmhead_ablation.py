@@ -1,6 +1,6 @@
 """What the fused lm_head kernel's time is made of: builds variants of csrc/ka_lmhead.hip with its LM_ABL_* switches
 (no slab copies / no fragment reads / no epilogue / copies that always hit L2 / no wait for the copies) and its copy
-schedule macros, times each at the BASELINE shape, and reports the shader clock each one ran at (the part is power
+schedule macros, times each at the headline shape (hidden [32768, 4096] x W [128256, 4096]), and reports the shader clock each one ran at (the part is power
 limited under this kernel, so a variant's time is cycles / clock with a clock that depends on what the variant does).
 
     python kernel-align_amd/benchmarks/lmhead_ablation.py [--sustained]

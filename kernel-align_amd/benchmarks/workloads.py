@@ -1,4 +1,4 @@
-"""Seeded input builders for the BASELINE configurations (shared by the benchmarks, the tests and the smoke check)."""
+"""Seeded input builders for the benchmark configurations (shared by the benchmarks, the tests and the smoke check)."""
 from __future__ import annotations
 
 import torch

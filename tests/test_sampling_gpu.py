@@ -2,7 +2,7 @@
 
 Token ids must be bit-exact against oracle/ka_oracle.c (the exactly specified definition) on
 every row, and against the torch restatement of the reference's native_sampling on every row
-whose threshold decisions are not within fp32 rounding noise of a tie (on the BASELINE
+whose threshold decisions are not within fp32 rounding noise of a tie (on the benchmark
 configuration that is every row).
 """
 import math
@@ -154,7 +154,7 @@ def test_every_bf16_value_through_the_temperature_step(sampler):
 def test_temperature_rule_against_torch_division_on_the_device(dtype):
     """The operator's temperature step is the true quotient round_dtype(float(x) / T) (what torch's CPU division
     returns, which is the oracle the parity target names).  torch's own GPU division by a Python scalar multiplies
-    by the fp32 reciprocal instead.  At the BASELINE temperature (0.7) and at 1.3 / 0.01 / 0.9 the two rules agree
+    by the fp32 reciprocal instead.  At the benchmark temperature (0.7) and at 1.3 / 0.01 / 0.9 the two rules agree
     on every finite 16-bit pattern; at e.g. 0.6 they differ on about 1.5 % of the patterns, which is recorded
     here so that a change of either side shows up."""
     bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype)
