@@ -15,7 +15,7 @@
 //     floor(u * Z_survivors).
 // The row is re-read by every pass; after the first it comes from L2 / MALL.
 // This radix path takes any row; shorter routes for common cases come first: the top-k candidate list
-// (ka_sampling_topk.h), and for 16-bit dtypes the no-filter and dense-histogram paths (ka_sampling_dense.h).
+// (ka_sampling_topk.h: top_k <= 1024), and for 16-bit dtypes the no-filter and dense-histogram paths (ka_sampling_dense.h).
 // For aligned fp32 rows outside the candidate list a variant of the kernel replaces the last pass by a draw
 // over shares of the row (ka_sampling_draw.h).
 #include <mutex>

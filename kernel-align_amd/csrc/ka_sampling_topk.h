@@ -1,4 +1,4 @@
-// Top-k fast path of the sampling kernel (1 <= top_k <= 1024): a short candidate list in LDS.
+// Top-k route of the sampling kernel (1 <= top_k <= 1024): a short candidate list in LDS.
 #ifndef KA_SAMPLING_TOPK_H
 #define KA_SAMPLING_TOPK_H
 
@@ -8,15 +8,19 @@ namespace ka {
 namespace {
 
 // ---------------------------------------------------------------------------
-// Top-k fast path: everything after the first read of the row happens on a short candidate list in LDS.
+// Top-k route: everything after the first read of the row happens on a short candidate list in LDS.
 //
-//   1. every lane takes the maximum raw key of its strided share of the row; the top_k-th largest of
-//      those 1024 maxima, t, is a lower bound of the top_k-th largest element;
+//   1. maxima of disjoint shares of the row are taken while it streams by (each maximum is a different element);
+//      the top_k-th largest of them, t, is a lower bound of the top_k-th largest element;
 //   2. the bound is lowered to the smallest raw key that still scales to the same value as t (ties made
-//      by the rounding of x / T must not be lost), and one more pass collects every element at or above
-//      it: a superset of the top-k survivors, ~top_k + a few entries on ordinary rows;
+//      by the rounding of x / T must not be lost), and every element at or above it is collected:
+//      a superset of the top-k survivors, ~top_k + a few entries on ordinary rows;
 //   3. the candidates are scaled, ranked by (key desc, index asc), cut by top-k (ties kept) and top-p on
 //      integer masses, and the draw is taken over the survivors in index order.
+// Two routes do this (fast_topk below chooses; the caller can force the second): the short route for top_k <= 256
+// (pooled maxima or a radix descent for the bound, candidate vectors re-read from L2, ranks by key and by index in one
+// step, a scan-based tail on one wavefront) and the block-wide route (radix descent, row kept in registers where it
+// fits, block-wide rank sort and scans).
 // Returns false (having written nothing) when the candidates do not fit: the radix path then runs.
 // All integer decisions are the same function of the row as in the radix path.
 // ---------------------------------------------------------------------------
