@@ -76,10 +76,11 @@ __device__ __forceinline__ uint32_t elem_key16(uint32_t raw, float temp) {
     return (h & 0x8000u) ? (~h & 0xffffu) : (h | 0x8000u);
 }
 
+// Sums over the 64 lanes of a wavefront (all lanes active), the total in every lane: a DPP prefix sum, then lane 63.
 __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    const uint64_t inc = wave_incl_scan_u64(v);
+    return (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc >> 32)), kWave - 1))) << 32) |
+           uint32_t(__builtin_amdgcn_readlane(int(uint32_t(inc)), kWave - 1));
 }
 __device__ __forceinline__ uint32_t block_max_u32_buf(uint32_t v, uint32_t *wave_buf) {
 #pragma unroll
@@ -392,21 +393,10 @@ __device__ __forceinline__ void for_wave_vectors(const uint4 *vp, int n_here, fl
 }
 
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    return uint32_t(__builtin_amdgcn_readlane(int(wave_incl_scan_u32(v)), kWave - 1));
 }
-// Exclusive prefix sums over the 64 lanes of a wavefront.
-template <typename V> __device__ __forceinline__ V wave_excl_scan(V v) {
-    const int lane = threadIdx.x & (kWave - 1);
-    V inc = v;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        const V t = __shfl_up(inc, off, kWave);
-        if (lane >= off) inc += t;
-    }
-    return inc - v;
-}
+// Exclusive prefix sums over the 64 lanes of a wavefront (all lanes active).
+template <typename V> __device__ __forceinline__ V wave_excl_scan(V v) { return wave_incl_scan(v) - v; }
 
 template <typename T, bool HAS_T, bool ALL_SURVIVE>
 __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename T::raw_t *rp, int vocab, bool vec,
