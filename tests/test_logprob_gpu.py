@@ -185,10 +185,22 @@ def test_full_size_grpo_group(sampler):
     assert torch.equal(flat, groups)
     assert torch.equal(flat, sampler.compute_logp(logits, ids, chunk_tokens=n_rows))
     assert torch.equal(flat, sampler.compute_logp(logits, ids, chunk_tokens=5000))
-    # oracle parity on three blocks (first, middle, last)
+    # oracle parity on three whole blocks (first, middle, last) and on every spike row of the tensor (found on the
+    # device: a spike is +25, N(0, 3^2) stays below 16): both branches of the spike closed form are hit, since every
+    # fourth spike row targets its spike
     for b in (0, 31, 63):
         s = b * blk
         lc, ic = logits[s:s + blk].cpu(), ids[s:s + blk].cpu()
         assert (flat[s:s + blk].cpu() - O.logprob_ref(lc, ic)).abs().max().item() <= TOL
+    spike_rows = torch.cat([(logits[s:s + blk].max(dim=-1).values.float() >= 24.0).nonzero().squeeze(-1) + s
+                            for s in range(0, n_rows, blk)])
+    assert 1000 <= spike_rows.numel() <= 1700                          # Bernoulli(0.01) of 131,072 rows
+    ls, isp = logits[spike_rows].cpu(), ids[spike_rows].cpu()
+    got_spike = flat[spike_rows].cpu()
+    assert (got_spike - O.logprob_ref(ls, isp)).abs().max().item() <= TOL
+    on_spike = ls.float().argmax(dim=-1) == isp
+    assert 200 <= int(on_spike.sum()) <= 500
+    lse_minus_c = math.log1p((vocab - 1) * math.exp(-25.0 + 4.5))      # crude bound: the rest of the row is exp(N(0, 9))
+    assert (got_spike[on_spike] > -lse_minus_c - 0.5).all() and (got_spike[on_spike] <= 0).all()
     # every row is a proper log-probability; spike rows that target their spike are ~0
     assert torch.isfinite(flat).all() and (flat <= 0).all()
