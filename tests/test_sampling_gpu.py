@@ -405,3 +405,17 @@ def test_masked_vocabulary_rows(sampler, dtype):
         got = check_exact(sampler, logits, u, k, p, temp)
         assert not masked[torch.arange(6), got[:6]].any()
         assert got[6] == 77
+
+
+def test_more_rows_than_compute_units(sampler):
+    """Batches beyond the 256 CUs of the part (several workgroups per CU in turn): ids against the oracle."""
+    g = torch.Generator().manual_seed(91)
+    logits = (torch.randn(1500, 4104, generator=g) * 3).bfloat16()
+    u = torch.rand(1500, generator=g)
+    for k, p, temp in ((50, 0.9, 0.7), (None, 0.9, 1.0), (None, None, 0.7), (300, None, 1.0)):
+        check_exact(sampler, logits, u, k, p, temp)
+    big, ub = cfg5_sampling(600)
+    got = run(sampler, big, ub, 50, 0.9, 0.7)
+    assert torch.equal(got[:64], exact.sample(big[:64], 0.7, 50, 0.9, ub[:64]))
+    assert torch.equal(got[-64:], exact.sample(big[-64:], 0.7, 50, 0.9, ub[-64:]))
+    assert torch.equal(got, torch.cat([run(sampler, big[s:s + 200], ub[s:s + 200], 50, 0.9, 0.7) for s in range(0, 600, 200)]))
