@@ -8,6 +8,10 @@ sampling_rows16.pt      16 bf16 rows of 4096 entries covering the edge cases (ti
                         tie at the top-p cut, all-equal, single spike, k >= V, masked prefix, -inf
                         only, signed zeros), with uniforms, (T, top_k, top_p) cases and the ids of
                         both sampling oracles.
+lmhead_extras.pt        hidden bf16 [40, 64] x W bf16 [500, 64] with ids: fp64 log-probabilities and entropies of the
+                        fused lm_head operator; bf16 logits [6, 777] with ids and upstream gradients: the fp64 gradient
+                        of the logprob operator (one row with a masked target); and the drawn token's log-probability
+                        of the sampling rows above for the first sampling case.
 Files hold tensors and plain Python scalars only; load them with torch.load(weights_only=True).
 """
 import math
@@ -59,6 +63,23 @@ def main():
         blob[f"ids_torch_{n}"] = ref_ids
         blob[f"margin_torch_{n}"] = margin
     torch.save(blob, HERE / "sampling_rows16.pt")
+    g = torch.Generator().manual_seed(123)
+    hidden = torch.randn(40, 64, generator=g).bfloat16()
+    weight = (torch.randn(500, 64, generator=g) * 0.2).bfloat16()
+    hid_ids = torch.randint(0, 500, (40,), generator=g)
+    full = torch.nn.functional.linear(hidden.double(), weight.double())
+    bl = (torch.randn(6, 777, generator=g) * 3).bfloat16()
+    bi = torch.randint(0, 777, (6,), generator=g)
+    bl[2, bi[2]] = -math.inf                             # a masked target: logp = -inf, finite gradient
+    bg = torch.randn(6, generator=g)
+    t0, k0, p0 = SAMPLING_CASES[0]
+    _, drawn_lp = exact.sample_rows(rows, t0, k0, p0, u)
+    torch.save({"hidden": hidden, "weight": weight, "ids": hid_ids,
+                "logp_f64": logprob_ref.lmhead_logprob_ref(hidden, weight, hid_ids, dtype=torch.float64),
+                "entropy_f64": logprob_ref.entropy_f64(full),
+                "bwd_logits": bl, "bwd_ids": bi, "bwd_grad": bg,
+                "bwd_dlogits_f64": logprob_ref.logprob_backward_closed_form(bl, bi, bg),
+                "drawn_logprob_case0": drawn_lp}, HERE / "lmhead_extras.pt")
     print("wrote", sorted(p.name for p in HERE.glob("*.pt")))
 
 

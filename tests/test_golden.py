@@ -52,3 +52,36 @@ def test_sampling_kernel_matches_fixture(sampler):
         assert torch.equal(got, b[f"ids_exact_{n}"]), n
         keep = torch.arange(16) != NAN_ROW
         assert torch.equal(got[keep], b[f"ids_torch_{n}"][keep]), n
+
+
+def test_extras_oracles_reproduce_fixture():
+    b = load("lmhead_extras.pt")
+    got = logprob_ref.lmhead_logprob_ref(b["hidden"], b["weight"], b["ids"], dtype=torch.float64)
+    assert torch.allclose(got, b["logp_f64"], atol=1e-13, rtol=0)
+    full = torch.nn.functional.linear(b["hidden"].double(), b["weight"].double())
+    assert torch.allclose(logprob_ref.entropy_f64(full), b["entropy_f64"], atol=1e-13, rtol=0)
+    d = logprob_ref.logprob_backward_closed_form(b["bwd_logits"], b["bwd_ids"], b["bwd_grad"])
+    assert torch.allclose(d, b["bwd_dlogits_f64"], atol=1e-14, rtol=0) and torch.isfinite(d).all()
+    s = load("sampling_rows16.pt")
+    n, t, k, p = next(sampling_cases(s))
+    _, lp = exact.sample_rows(s["logits"], t, k, p, s["uniforms"])
+    assert torch.equal(lp, b["drawn_logprob_case0"])
+
+
+@pytest.mark.gpu
+def test_extras_kernels_match_fixture(sampler):
+    b = load("lmhead_extras.pt")
+    lp, ent = sampler.fused_linear_logp(b["hidden"].cuda(), b["weight"].cuda(), b["ids"].cuda(), return_entropy=True)
+    assert (lp.cpu().double() - b["logp_f64"]).abs().max().item() <= 1e-4
+    assert (ent.cpu().double() - b["entropy_f64"]).abs().max().item() <= 1e-4
+    logits, ids, grad = b["bwd_logits"].cuda(), b["bwd_ids"].cuda(), b["bwd_grad"].cuda()
+    logp = sampler.compute_logp(logits, ids)
+    d = sampler.compute_logp_backward(logits, ids, logp, grad).cpu().double()
+    want = b["bwd_dlogits_f64"]
+    assert ((d - want).abs() <= 2.0 ** -8 * want.abs() + 1e-6).all()
+    s = load("sampling_rows16.pt")
+    n, t, k, p = next(sampling_cases(s))
+    ids2, lp2 = sampler.sample(s["logits"].cuda(), top_k=k, top_p=p, temperature=t, uniforms=s["uniforms"].cuda(),
+                               return_logprob=True)
+    assert torch.equal(ids2.cpu(), s[f"ids_exact_{n}"])
+    assert (lp2.cpu().double() - b["drawn_logprob_case0"]).abs().max().item() <= 1e-5
