@@ -942,6 +942,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         }
     }
     __syncthreads();
+    KA_STAMP(13);  // masses of every share
     // 7b. the segment (a wavefront's share, or the tail) that holds floor(u * Z)
     uint64_t z = 0;
     {
@@ -1068,6 +1069,7 @@ __device__ __forceinline__ bool dense_stream(unsigned char *lds, const typename 
         }
     }
     __syncthreads();
+    KA_STAMP(14);  // entry located
     if (tid == 0) {
         *out_slot = ds.hit;
         if (lp_slot != nullptr) *lp_slot = ds.hit >= 0 ? log_ratio(ds.pick_w, z) : __builtin_nanf("");
