@@ -38,10 +38,9 @@ class RolloutExecutor:
     def step(self, logits, uniforms=None):
         """One decode step: sample a token per row of `logits` [B, V] and return (ids, logprobs)."""
         sample = kernel_registry.resolve("sampling")
-        logp = kernel_registry.resolve("fused_logp")
-        ids = sample(logits, top_k=self.config.get("top_k"), top_p=self.config.get("top_p"),
-                     temperature=self.config.get("temperature", 1.0), uniforms=uniforms)
-        return ids, logp(logits, ids)
+        # both kernels from one operator call: at small batches the host time of a call exceeds the kernels' time
+        return sample(logits, top_k=self.config.get("top_k"), top_p=self.config.get("top_p"),
+                      temperature=self.config.get("temperature", 1.0), uniforms=uniforms, return_policy_logprob=True)
 
     def generate(self, next_logits: Callable, prompt_ids, max_new_tokens: int, uniforms=None,
                  eos_id: Optional[int] = None):

@@ -47,9 +47,9 @@ class GraphedDecodeStep:
             self.ids, self.logp = self._run()
 
     def _run(self):
-        ids = self.sampler.sample(self.logits, uniforms=self.uniforms, **self._kw)
-        logp = self.sampler.compute_logp(self.logits, ids) if self._with_logprob else None
-        return ids, logp
+        if self._with_logprob:
+            return self.sampler.sample(self.logits, uniforms=self.uniforms, return_policy_logprob=True, **self._kw)
+        return self.sampler.sample(self.logits, uniforms=self.uniforms, **self._kw), None
 
     def __call__(self, logits=None, uniforms=None):
         """Replay the step.  `logits` / `uniforms`, if given, are copied into the step's input buffers first."""

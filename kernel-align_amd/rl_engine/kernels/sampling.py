@@ -272,7 +272,7 @@ class SamplerBackend(nn.Module):
     # ----------------------------------------------------------------- sampling
     @torch.inference_mode()
     def sample(self, logits, top_k=None, top_p=None, temperature=1.0, deterministic=True,
-               uniforms=None, generator=None, return_logprob=False, route_flags=0):
+               uniforms=None, generator=None, return_logprob=False, route_flags=0, return_policy_logprob=False):
         """Draw one token id per row after temperature -> top-k -> top-p filtering.
 
         logits: [B, V] bf16 / fp16 / fp32 on the GPU.  Returns int64 [B] (reference:
@@ -286,6 +286,10 @@ class SamplerBackend(nn.Module):
         is ``(ids, logprob)`` where logprob (fp32 [B]) is the log-probability of the drawn token under the
         filtered, renormalised distribution it was drawn from.  ``route_flags`` (``_hip.SAMPLE_FLAG_*``) makes the
         library take one of its slower routes for the same function; results do not depend on it.
+        With ``return_policy_logprob=True`` the last element of the result is the drawn token's log-probability
+        under the unfiltered softmax of the raw logits - ``compute_logp(logits, ids)``, what a GRPO ratio is built
+        from - enqueued behind the sampling kernel from this same call (a decode step then costs one operator call
+        of host time instead of two).
         """
         _require_gpu(logits, "logits")
         if logits.dim() != 2:
@@ -330,6 +334,9 @@ class SamplerBackend(nn.Module):
         out = torch.empty(batch, dtype=torch.int64, device=dev)
         logprob = torch.empty(batch, dtype=torch.float32, device=dev) if return_logprob else None
         if batch == 0:
+            empty = torch.empty(0, dtype=torch.float32, device=dev)
+            if return_policy_logprob:
+                return (out, logprob, empty) if return_logprob else (out, empty)
             return (out, logprob) if return_logprob else out
         ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
         row_stride = rows.stride(0) if batch > 1 else vocab
@@ -353,7 +360,15 @@ class SamplerBackend(nn.Module):
             else:
                 with self._workspace(ws_bytes, dev) as ws_ptr:
                     fn_name, status = launch(ws_ptr)
+            policy = None
+            if status == _hip.KA_OK and return_policy_logprob:
+                policy = torch.empty(batch, dtype=torch.float32, device=dev)
+                fn_name = _LOGPROB_FN[logits.dtype]
+                status = getattr(self._lib, fn_name)(rows.data_ptr(), batch, vocab, row_stride, out.data_ptr(),
+                                                     policy.data_ptr(), _raw_stream())
         _hip.check(status, fn_name)
+        if return_policy_logprob:
+            return (out, logprob, policy) if return_logprob else (out, policy)
         return (out, logprob) if return_logprob else out
 
     # ---------------------------------------------------------------- fused GEMM

@@ -125,3 +125,23 @@ def test_decode_step_replayed_from_a_hip_graph(sampler):
         assert torch.equal(got_ids, eager_ids) and torch.equal(got_logp, eager_logp)
         assert torch.equal(got_ids.cpu(), exact.sample(logits, 0.7, 50, 0.9, u))
         assert (got_logp.cpu() - logprob_ref.logprob_ref(logits, got_ids.cpu())).abs().max().item() <= 1e-4
+
+
+def test_policy_logprob_from_the_sampling_call(sampler):
+    """sample(..., return_policy_logprob=True) enqueues the logprob kernel behind the sampling kernel: the same bits
+    as a separate compute_logp call, alone and together with the filtered-distribution log-probability."""
+    g = torch.Generator().manual_seed(81)
+    for dtype in (torch.bfloat16, torch.float32):
+        logits = (torch.randn(40, 9000, generator=g) * 3).to(dtype).cuda()
+        u = torch.rand(40, generator=g).cuda()
+        ids, policy = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+        assert torch.equal(ids, sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u))
+        assert torch.equal(policy, sampler.compute_logp(logits, ids))
+        ids2, lp, policy2 = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_logprob=True,
+                                           return_policy_logprob=True)
+        assert torch.equal(ids2, ids) and torch.equal(policy2, policy) and (lp <= 0).all()
+        # without a temperature the filters only remove mass: the drawn token's filtered probability is at least its policy one
+        _, lp1, pol1 = sampler.sample(logits, top_k=50, top_p=0.9, uniforms=u, return_logprob=True, return_policy_logprob=True)
+        assert (lp1 >= pol1 - 1e-5).all()
+    e_ids, e_pol = sampler.sample(torch.empty(0, 100, dtype=torch.bfloat16, device="cuda"), return_policy_logprob=True)
+    assert e_ids.numel() == 0 and e_pol.numel() == 0
