@@ -153,6 +153,11 @@ int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, in
  * log(mass of the sampled entry / total surviving mass), the log-probability under the distribution the
  * entry was drawn from.  The reference takes scalars only (rl_engine/kernels/sampling.py:39); the
  * FlashInfer operators it forwards to accept per-row tensors (sampling.py:62-64).
+ * out_policy_logprob (optional, fp32 [batch]) receives the sampled entry's log-probability under the unfiltered
+ * softmax of the raw logits, logits[r, id] - logsumexp(logits[r, :]): what ka_logprob_* returns for it (to 1e-5:
+ * the sum runs over the row in another fixed order) and what a GRPO ratio is built from.  With top_k <= 256 the
+ * log-sum-exp is taken along while the row streams by (a decode step then needs no second kernel); the other
+ * routes pass over the row once more at their end.
  * flags (0 in production) selects among routes that compute the same function, so that a caller can check one
  * against the other: KA_SAMPLE_FLAG_GENERAL_PATH runs the general radix-select path even where a shorter route
  * applies; KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK keeps the top-k route on its block-wide selection and tail instead of the
@@ -163,7 +168,8 @@ int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, in
 int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                  float temperature, const float *temperature_rows, int32_t top_k, const int32_t *top_k_rows,
                  float top_p, const float *top_p_rows, const float *uniforms, int64_t *out_ids,
-                 float *out_logprob, uint32_t flags, void *workspace, size_t workspace_bytes, void *hip_stream);
+                 float *out_logprob, float *out_policy_logprob, uint32_t flags, void *workspace,
+                 size_t workspace_bytes, void *hip_stream);
 
 /*
  * The integer mass function of the sampling operator, element-wise: out[i] = W(d[i]) =

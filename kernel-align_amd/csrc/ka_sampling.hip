@@ -41,6 +41,7 @@ struct SampleParams {
     const float *uniforms;
     int64_t *out_ids;
     float *out_logprob;  // optional: log of the sampled entry's probability under the filtered distribution
+    float *out_policy;   // optional: its log-probability under the unfiltered softmax of the raw logits
 };
 
 // ---------------------------------------------------------------------------
@@ -58,10 +59,11 @@ template <bool DENSE> __device__ __forceinline__ unsigned char *lds_base() {
     }
 }
 
+// One row.  Returns 1 when the row's id (and filtered log-probability) is written or on its way (on some routes one
+// wavefront still finishes while the others return), 2 when the same holds for the policy log-probability.
 template <typename T, bool DENSE>
-__global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t *__restrict__ logits,
-                                                         int vocab, int64_t row_stride, SampleParams prm, int vec,
-                                                         int no_fast) {
+__device__ __forceinline__ int sample_one_row(const typename T::raw_t *__restrict__ logits, int vocab, int64_t row_stride,
+                                              const SampleParams &prm, int vec, int no_fast, PolicyLse &lse) {
     constexpr int EPV = T::kPerVec;
     constexpr int LEVELS = Round<T>::kLevels;
     // For fp32 rows the second variant is the radix path alone, with the draw done by shares of the row; the host
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (prm.top_k_rows != nullptr) { top_k = prm.top_k_rows[row]; if (top_k < 0) top_k = 0; }
     if (prm.top_p_rows != nullptr) { top_p = prm.top_p_rows[row]; if (!(top_p > 0.0f && top_p <= 1.0f)) top_p = 1.0f; }
     const float *__restrict__ uniforms = prm.uniforms;
-    int64_t *__restrict__ out = prm.out_ids;
+    int64_t *out = prm.out_ids;  // (not restrict: the kernel reads the id back through prm.out_ids for the policy log-probability)
     float *lp_slot = prm.out_logprob != nullptr ? prm.out_logprob + row : nullptr;
     const bool has_t = temp != 1.0f;
     const bool use_k = top_k > 0 && top_k < vocab;
@@ -94,9 +96,9 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     // no_fast: bit 0 = take the general radix path, bit 1 = keep the top-k route block-wide (KA_SAMPLE_FLAG_*)
     if (!RADIX_ONLY && use_k && top_k <= S_THREADS && !(no_fast & 1)) {
         if constexpr (!RADIX_ONLY) {
-            if (fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot,
-                             (no_fast & 2) != 0))
-                return;
+            const int done = fast_topk<T>(sh, rp, vocab, vec, temp, has_t, top_k, use_p, top_p, u, out + row, lp_slot,
+                                          (no_fast & 2) != 0, prm.out_policy != nullptr ? prm.out_policy + row : nullptr, lse);
+            if (done) return done;
         }
         __syncthreads();
     } else if (!(no_fast & 1)) {
@@ -110,12 +112,12 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
                                                             out + row, lp_slot)
                              : dense_stream<T, false, false>(lds, rp, vocab, vec, temp, use_k, top_k, use_p, top_p, u,
                                                              out + row, lp_slot);
-            if (done) return;
+            if (done) return 1;
             __syncthreads();
         }
         if constexpr (!DENSE && T::kBytes == 2) {
             if (!use_k && !use_p) {  // launched without the histogram's LDS: fp16, whose rows hold too many distinct values
-                if (nofilter_resident<T>(sh.ds, rp, vocab, vec, temp, has_t, u, out + row, lp_slot)) return;
+                if (nofilter_resident<T>(sh.ds, rp, vocab, vec, temp, has_t, u, out + row, lp_slot)) return 1;
                 __syncthreads();
             }
         }
@@ -248,7 +250,7 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if constexpr (RADIX_ONLY) {
         if (vec) {
             draw_by_shares<T>(sh.ds, rp, vocab, temp, has_t, kmax, vmax, kcut, r_cut, u, out + row, lp_slot);
-            return;
+            return 1;
         }
     }
     const uint64_t tau = floor_scale(u, z_kept);
@@ -308,6 +310,27 @@ __global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t
     if (tid == 0) {
         out[row] = sh.hit;
         if (lp_slot != nullptr) *lp_slot = sh.hit >= 0 ? log_ratio(sh.pick_z, z_kept) : __builtin_nanf("");
+    }
+    return 1;
+}
+
+template <typename T, bool DENSE>
+__global__ __launch_bounds__(S_THREADS) void sample_rows(const typename T::raw_t *__restrict__ logits,
+                                                         int vocab, int64_t row_stride, SampleParams prm, int vec,
+                                                         int no_fast) {
+    // per-wavefront partial results of the row's log-sum-exp (its own few bytes of LDS: the routes' memory may still be
+    // in use by a wavefront that finishes the row)
+    __shared__ PolicyLse lse;
+    const int done = sample_one_row<T, DENSE>(logits, vocab, row_stride, prm, vec, no_fast, lse);
+    if (prm.out_policy != nullptr && done != 2) {
+        // The route did not take the log-sum-exp along: one more pass over the row (from L2), by the whole block.
+        const int64_t row = blockIdx.x;
+        const typename T::raw_t *rp = logits + row * row_stride;
+        LaneLse acc;
+        for_each_raw<T>(rp, vocab, vec != 0, [&](int, typename T::raw_t raw) { acc.add(T::widen(raw)); });
+        acc.to_block(lse);
+        __syncthreads();  // also: the id of the row is written (by thread 0, or by the wavefront that finished the row)
+        if (threadIdx.x == 0) prm.out_policy[row] = lse.finish<T>(rp, prm.out_ids[row], vocab);
     }
 }
 
@@ -472,12 +495,13 @@ KA_EXPORT int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, voi
 KA_EXPORT int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                            float temperature, const float *temperature_rows, int32_t top_k,
                            const int32_t *top_k_rows, float top_p, const float *top_p_rows, const float *uniforms,
-                           int64_t *out_ids, float *out_logprob, uint32_t flags, void *workspace,
-                           size_t workspace_bytes, void *hip_stream) {
+                           int64_t *out_ids, float *out_logprob, float *out_policy_logprob, uint32_t flags,
+                           void *workspace, size_t workspace_bytes, void *hip_stream) {
     ka::SampleParams p = ka::scalar_params(temperature, top_k, top_p, uniforms, out_ids);
     p.temperature_rows = temperature_rows;
     p.top_k_rows = top_k_rows;
     p.top_p_rows = top_p_rows;
     p.out_logprob = out_logprob;
+    p.out_policy = out_policy_logprob;
     return ka::launch_ex(dtype, logits, batch, vocab, row_stride, p, workspace, workspace_bytes, hip_stream, flags);
 }

@@ -288,6 +288,69 @@ __device__ __forceinline__ void clear_hist(Shared &sh) {
 }
 
 // ---------------------------------------------------------------------------
+// Log-sum-exp of the raw row, taken along by the sampling kernel when the caller wants the drawn token's
+// log-probability under the unfiltered softmax (what the logprob operator returns for it).  A lane folds its
+// elements online in fp32 (base-2 exponentials relative to a running maximum), the lanes of a wavefront are folded by
+// a fixed butterfly, the wavefronts in wavefront order: the value depends on the row and on the route its sampling
+// takes, not on the batch.
+// ---------------------------------------------------------------------------
+constexpr float kLseLog2e = 1.44269504088896340736f;
+constexpr float kLseFloor = -1.0e30f;  // running maxima start here: (old max - new max) is never inf - inf
+
+struct PolicyLse {  // in LDS
+    float wave_ml2[S_WAVES];  // maximum * log2(e) of each wavefront's elements
+    float wave_s[S_WAVES];    // sum of 2^(x * log2(e) - wave_ml2)
+    // log-probability of element `hit` of the row (thread 0, after a barrier behind to_block)
+    template <typename T> __device__ __forceinline__ float finish(const typename T::raw_t *rp, int64_t hit, int vocab) const {
+        if (hit < 0 || hit >= vocab) return __builtin_nanf("");
+        float big = wave_ml2[0];
+#pragma unroll
+        for (int w = 1; w < S_WAVES; ++w) big = fmaxf(big, wave_ml2[w]);
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < S_WAVES; ++w) total += wave_s[w] * fast_exp2(wave_ml2[w] - big);
+        const double lse = (double(big) + log2(double(total))) * 0.693147180559945309417232;
+        return float(double(T::widen(rp[hit])) - lse);
+    }
+};
+
+struct LaneLse {
+    float m = kLseFloor, ml2 = kLseFloor * kLseLog2e, s = 0.0f;
+    // Contraction is off in these functions: fused into an FMA against the fresh product, (ml2 - mn * log2e) would return
+    // the rounding residue of a 1e30-sized product instead of 0 while the maximum still sits at the floor, and 2^residue
+    // overflows.
+    __device__ __forceinline__ void add(float x) {
+#pragma clang fp contract(off)
+        const float mn = fmaxf(m, x);
+        const float ml2n = mn * kLseLog2e;
+        s = fmaf(s, fast_exp2(ml2 - ml2n), fast_exp2(fmaf(x, kLseLog2e, -ml2n)));
+        m = mn;
+        ml2 = ml2n;
+    }
+    // N elements whose maximum vm is known already: one rescale for all of them
+    template <int N> __device__ __forceinline__ void add_vector(const float (&x)[N], float vm) {
+#pragma clang fp contract(off)
+        const float mn = fmaxf(m, vm);
+        const float ml2n = mn * kLseLog2e;
+        float e = 0.0f;
+#pragma unroll
+        for (int j = 0; j < N; ++j) e += fast_exp2(fmaf(x[j], kLseLog2e, -ml2n));
+        s = fmaf(s, fast_exp2(ml2 - ml2n), e);
+        m = mn;
+        ml2 = ml2n;
+    }
+    // every thread of the block calls this; a barrier must follow before PolicyLse::finish
+    __device__ __forceinline__ void to_block(PolicyLse &out) const {
+        const float wm = wave_max(ml2);
+        const float ws = wave_sum(s * fast_exp2(ml2 - wm));
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            out.wave_ml2[threadIdx.x / kWave] = wm;
+            out.wave_s[threadIdx.x / kWave] = ws;
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------
 // Row traversal: f(index, raw element) for every element, any order.
 // ---------------------------------------------------------------------------
 template <typename T, int U = 4, typename F>

@@ -66,7 +66,8 @@ static_assert(2 * SHORT_CAND <= CAND_CAP && SHORT_VECS * 16 <= CAND_CAP * 8, "th
 // as the block-wide tail, without a barrier and without a loop over pairs.
 template <typename T, int SLOTS>
 __device__ __forceinline__ void short_tail(Shared &sh, uint32_t nc, uint32_t na, const uint32_t *rank_by_index,
-                                           bool use_p, float top_p, float u, int64_t *out_slot, float *lp_slot) {
+                                           bool use_p, float top_p, float u, int64_t *out_slot, float *lp_slot,
+                                           const typename T::raw_t *rp, int vocab, float *policy_slot, const PolicyLse &lse) {
     const int lane = threadIdx.x & (kWave - 1);
     uint64_t w[SLOTS], before[SLOTS];
     uint64_t carry = 0;
@@ -132,13 +133,17 @@ __device__ __forceinline__ void short_tail(Shared &sh, uint32_t nc, uint32_t na,
     if (lane == 0) {
         *out_slot = hit == 0xffffffffu ? int64_t(-1) : int64_t(hit);
         if (lp_slot != nullptr) *lp_slot = hit == 0xffffffffu ? __builtin_nanf("") : log_ratio(w_hit, z_kept);
+        if (policy_slot != nullptr) *policy_slot = lse.template finish<T>(rp, hit == 0xffffffffu ? int64_t(-1) : int64_t(hit), vocab);
     }
 }
 
+// Returns 0 (nothing written: the radix path runs), 1 (id and filtered log-probability written) or 2 (the policy
+// log-probability as well: the short route takes the row's log-sum-exp along while the row streams by).
 template <typename T>
-__device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *rp, int vocab, bool vec, float temp,
-                                          bool has_t, int top_k, bool use_p, float top_p, float u,
-                                          int64_t *out_slot, float *lp_slot, bool block_wide_only) {
+__device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp, int vocab, bool vec, float temp,
+                                         bool has_t, int top_k, bool use_p, float top_p, float u,
+                                         int64_t *out_slot, float *lp_slot, bool block_wide_only, float *policy_slot,
+                                         PolicyLse &lse) {
     const int tid = threadIdx.x;
     // top_k <= 64 takes the short route unless the caller asks for the block-wide one (the two give the same ids)
     const bool short_route = top_k <= SHORT_TOPK && !block_wide_only;
@@ -166,6 +171,9 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     const int trk_need = (nvec + TRK_VECS * S_THREADS - 1) / (TRK_VECS * S_THREADS);
     const int trk_rounds = T::kBytes == 4 ? trk_need : 1;
     const bool tracked = vec && !resident && trk_need <= (T::kBytes == 4 ? 4 : 1);
+    // the short route folds the row's log-sum-exp while it reads the row (it never keeps the row in registers)
+    const bool take_lse = short_route && policy_slot != nullptr;
+    LaneLse acc_lse;
     uint4 held[RES_VECS];
     // The slot maxima of a 16-bit row are kept in the row's own 16 bits, two per register (they are elements of the
     // row, so nothing is lost): 32 floats next to the loads in flight would spill.
@@ -222,14 +230,24 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
 #pragma unroll
                 for (int s = 0; s < TRK_BATCH; ++s) {
                     float vm = -__builtin_inff();
-                    if (base + (g * TRK_BATCH + s) * S_THREADS < nvec) vm = vector_max(q[s]);
+                    if (base + (g * TRK_BATCH + s) * S_THREADS < nvec) {
+                        vm = vector_max(q[s]);
+                        if (take_lse) {
+                            float x[EPV];
+                            T::unpack(q[s], x);
+                            acc_lse.add_vector(x, vm);
+                        }
+                    }
                     set_slot_max(g * TRK_BATCH + s, vm, round == 0);
                     lmaxf = fmaxf(lmaxf, vm);
                 }
             }
         }
         const int i = nvec * EPV + tid;  // ragged tail of the row
-        if (i < vocab) lmaxf = fmaxf(lmaxf, T::widen(rp[i]));
+        if (i < vocab) {
+            lmaxf = fmaxf(lmaxf, T::widen(rp[i]));
+            if (take_lse) acc_lse.add(T::widen(rp[i]));
+        }
     } else if (resident) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll
@@ -248,8 +266,12 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
         const int i = nvec * EPV + tid;  // ragged tail of the row
         if (i < vocab) lmaxf = fmaxf(lmaxf, T::widen(rp[i]));
     } else {
-        for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) { lmaxf = fmaxf(lmaxf, T::widen(raw)); });
+        for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) {
+            lmaxf = fmaxf(lmaxf, T::widen(raw));
+            if (take_lse) acc_lse.add(T::widen(raw));
+        });
     }
+    if (take_lse) acc_lse.to_block(lse);  // a barrier follows on every way on (pooling of the maxima, radix descent)
     KA_STAMP(1);   // row read, lane maxima known
     // 2. (both routes) the bound is widened over the raw values that scale to the same value; false: a huge
     //    temperature folds too many values together
@@ -331,12 +353,12 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
             __syncthreads();
         }
         KA_STAMP(2);   // bound known
-        if (!widen_bound(bound)) return false;
+        if (!widen_bound(bound)) return 0;
         KA_STAMP(3);   // bound widened
         const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
         // Fewer than top_k groups hold a number above -inf: the survivors may include -inf entries (and NaNs, which
         // count as -inf but fail every float compare).  Leave such rows to the radix path.
-        if (boundf == -__builtin_inff()) return false;
+        if (boundf == -__builtin_inff()) return 0;
         // S3. Vectors that hold a candidate go to a list in LDS whole (one atomic per vector, nothing per element
         //     in the wavefronts that hold the row); single elements (ragged tail, unaligned rows) go straight to the
         //     candidate list with their scaled key.
@@ -400,7 +422,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
             __syncthreads();
             KA_STAMP(10);  // candidates expanded
             const uint32_t nc = sh.n_cand;
-            if (nc > CAND_CAP) return false;
+            if (nc > CAND_CAP) return 0;
             if (nc <= uint32_t(SHORT_CAND)) {
                 // S5. Four threads rank one candidate twice, by (scaled key descending, index ascending) and by index
                 //     alone, and file it under both ranks together with its integer mass (see by_index_w above; none
@@ -462,13 +484,13 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
                         const uint32_t pp = uint32_t(s * kWave + tid);
                         na += uint32_t(__popcll(__ballot(pp < nc && sh.c.raw[pp] >= kstar)));
                     }
-                    if (na <= uint32_t(kWave)) short_tail<T, 1>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
-                    else if (na <= uint32_t(2 * kWave)) short_tail<T, 2>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
-                    else if (na <= uint32_t(4 * kWave)) short_tail<T, 4>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
-                    else short_tail<T, 8>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot);
+                    if (na <= uint32_t(kWave)) short_tail<T, 1>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot, rp, vocab, take_lse ? policy_slot : nullptr, lse);
+                    else if (na <= uint32_t(2 * kWave)) short_tail<T, 2>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot, rp, vocab, take_lse ? policy_slot : nullptr, lse);
+                    else if (na <= uint32_t(4 * kWave)) short_tail<T, 4>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot, rp, vocab, take_lse ? policy_slot : nullptr, lse);
+                    else short_tail<T, 8>(sh, nc, na, rank_by_index, use_p, top_p, u, out_slot, lp_slot, rp, vocab, take_lse ? policy_slot : nullptr, lse);
                     KA_STAMP(9);
                 }
-                return true;
+                return take_lse ? 2 : 1;
             }
             have_candidates = true;  // more than 512 candidates (a large tie group): the block-wide tail ranks them
         }
@@ -479,12 +501,12 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     if (tid == 0) { sh.n_cand = 0; sh.hit = -1; }
     __syncthreads();
     KA_STAMP(2);   // bound known
-    if (!widen_bound(bound)) return false;
+    if (!widen_bound(bound)) return 0;
     KA_STAMP(3);   // bound widened
     const float boundf = value_of<T>(bound);  // a float compare admits -0 next to +0: still a superset
     // Fewer than top_k lanes hold a number above -inf: the survivors then include -inf entries (and NaNs,
     // which count as -inf but fail every float compare).  Leave such rows to the radix path.
-    if (boundf == -__builtin_inff()) return false;
+    if (boundf == -__builtin_inff()) return 0;
     auto collect = [&](int i, typename T::raw_t raw) {
         if (T::widen(raw) >= boundf) {
             const uint32_t slot = atomicAdd(&sh.n_cand, 1u);
@@ -531,7 +553,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     KA_STAMP(4);   // candidates collected
     }
     const uint32_t nc = sh.n_cand;
-    if (nc > CAND_CAP) return false;
+    if (nc > CAND_CAP) return 0;
     // 3a. scale the candidates and rank them by (key desc, index asc)
     uint32_t my_key = 0, my_idx = 0;
     if (tid < int(nc)) {
@@ -620,7 +642,7 @@ __device__ __forceinline__ bool fast_topk(Shared &sh, const typename T::raw_t *r
     KA_STAMP(9);
     if (tid == 0) *out_slot = sh.hit;
     if (lp_slot != nullptr && tid < int(nb) && int64_t(sh.c.sidx[tid]) == sh.hit) *lp_slot = log_ratio(sh.c.w[tid], z_kept);
-    return true;
+    return 1;
 }
 
 

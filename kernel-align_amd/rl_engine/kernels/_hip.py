@@ -46,7 +46,7 @@ SIGNATURES = {
     "ka_sample_topk_topp_f16": (c_int, _SAMPLE_ARGS),
     "ka_sample_topk_topp_f32": (c_int, _SAMPLE_ARGS),
     "ka_sample_ex": (c_int, [c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_int32, c_void_p, c_float,
-                             c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_size_t, c_void_p]),
+                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_size_t, c_void_p]),
     "ka_sample_mass_fixed": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "ka_lmhead_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "ka_lmhead_logprob_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,

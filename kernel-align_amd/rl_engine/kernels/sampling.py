@@ -287,9 +287,9 @@ class SamplerBackend(nn.Module):
         filtered, renormalised distribution it was drawn from.  ``route_flags`` (``_hip.SAMPLE_FLAG_*``) makes the
         library take one of its slower routes for the same function; results do not depend on it.
         With ``return_policy_logprob=True`` the last element of the result is the drawn token's log-probability
-        under the unfiltered softmax of the raw logits - ``compute_logp(logits, ids)``, what a GRPO ratio is built
-        from - enqueued behind the sampling kernel from this same call (a decode step then costs one operator call
-        of host time instead of two).
+        under the unfiltered softmax of the raw logits - ``compute_logp(logits, ids)`` to 1e-5, what a GRPO ratio is
+        built from - computed by the sampling kernel itself (with ``top_k <= 256`` while the row streams by), so that
+        a decode step needs neither a second operator call nor a second kernel.
         """
         _require_gpu(logits, "logits")
         if logits.dim() != 2:
@@ -340,14 +340,16 @@ class SamplerBackend(nn.Module):
             return (out, logprob) if return_logprob else out
         ws_bytes = self._lib.ka_sample_workspace_bytes(batch, vocab)
         row_stride = rows.stride(0) if batch > 1 else vocab
-        extended = return_logprob or k_rows is not None or p_rows is not None or t_rows is not None or route_flags
+        extended = (return_logprob or return_policy_logprob or k_rows is not None or p_rows is not None
+                    or t_rows is not None or route_flags)
+        policy = torch.empty(batch, dtype=torch.float32, device=dev) if return_policy_logprob else None
         def launch(ws_ptr):
             stream = _raw_stream()
             if extended:
                 ptr = lambda x: None if x is None else x.data_ptr()  # noqa: E731
                 return "ka_sample_ex", self._lib.ka_sample_ex(
                     _DTYPE_CODE[logits.dtype], rows.data_ptr(), batch, vocab, row_stride, t, ptr(t_rows), k,
-                    ptr(k_rows), p, ptr(p_rows), uniforms.data_ptr(), out.data_ptr(), ptr(logprob),
+                    ptr(k_rows), p, ptr(p_rows), uniforms.data_ptr(), out.data_ptr(), ptr(logprob), ptr(policy),
                     int(route_flags), ws_ptr, ws_bytes, stream)
             name = _SAMPLE_FN[logits.dtype]
             return name, getattr(self._lib, name)(
@@ -360,12 +362,6 @@ class SamplerBackend(nn.Module):
             else:
                 with self._workspace(ws_bytes, dev) as ws_ptr:
                     fn_name, status = launch(ws_ptr)
-            policy = None
-            if status == _hip.KA_OK and return_policy_logprob:
-                policy = torch.empty(batch, dtype=torch.float32, device=dev)
-                fn_name = _LOGPROB_FN[logits.dtype]
-                status = getattr(self._lib, fn_name)(rows.data_ptr(), batch, vocab, row_stride, out.data_ptr(),
-                                                     policy.data_ptr(), _raw_stream())
         _hip.check(status, fn_name)
         if return_policy_logprob:
             return (out, logprob, policy) if return_logprob else (out, policy)

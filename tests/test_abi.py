@@ -62,14 +62,14 @@ def test_sampling_argument_checks():
     assert call(p, 2, 1 << 22, 1 << 22, 1.0, 5, 0.9, p, p, None, 0, None) == _hip.KA_ERR_UNSUPPORTED
     assert lib.ka_sample_workspace_bytes(256, 128256) >= 0
     ex = lib.ka_sample_ex
-    assert ex(0, None, 0, 128, 128, 1.0, None, 0, None, 1.0, None, None, None, None, 0, None, 0, None) == _hip.KA_OK
-    assert ex(7, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG   # dtype code
-    assert ex(0, p, 2, 128, 128, 0.0, None, 0, None, 1.0, None, p, p, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG   # scalar T
-    assert ex(0, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, 4, None, 0, None) == _hip.KA_ERR_BAD_ARG   # flag bits
+    assert ex(0, None, 0, 128, 128, 1.0, None, 0, None, 1.0, None, None, None, None, None, 0, None, 0, None) == _hip.KA_OK
+    assert ex(7, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG   # dtype code
+    assert ex(0, p, 2, 128, 128, 0.0, None, 0, None, 1.0, None, p, p, None, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG   # scalar T
+    assert ex(0, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 4, None, 0, None) == _hip.KA_ERR_BAD_ARG   # flag bits
     assert b"flag" in lib.ka_last_error()
     # a per-row array replaces its scalar, which is then not checked: the call gets past the scalar checks and
     # is stopped by the next host check (stride < vocab), so nothing is ever launched on these made-up pointers
-    assert ex(0, p, 2, 128, 64, 0.0, p, -1, p, 9.0, p, p, p, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG
+    assert ex(0, p, 2, 128, 64, 0.0, p, -1, p, 9.0, p, p, p, None, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG
     assert b"stride" in lib.ka_last_error()
 
 

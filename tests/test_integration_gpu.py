@@ -118,8 +118,9 @@ def test_decode_step_replayed_from_a_hip_graph(sampler):
             ids, logp = step()
         got_ids, got_logp = ids.clone(), logp.clone()
         torch.cuda.synchronize()
-        eager_ids = sampler.sample(logits.cuda(), top_k=50, top_p=0.9, temperature=0.7, uniforms=u.cuda())
-        eager_logp = sampler.compute_logp(logits.cuda(), eager_ids)
+        eager_ids, eager_logp = sampler.sample(logits.cuda(), top_k=50, top_p=0.9, temperature=0.7, uniforms=u.cuda(),
+                                               return_policy_logprob=True)
+        assert (eager_logp - sampler.compute_logp(logits.cuda(), eager_ids)).abs().max().item() <= 1e-5
         junk = torch.randn(1 << 20, device="cuda").sum().item()          # eager work and a sync between replays
         assert junk == junk
         assert torch.equal(got_ids, eager_ids) and torch.equal(got_logp, eager_logp)
@@ -128,20 +129,41 @@ def test_decode_step_replayed_from_a_hip_graph(sampler):
 
 
 def test_policy_logprob_from_the_sampling_call(sampler):
-    """sample(..., return_policy_logprob=True) enqueues the logprob kernel behind the sampling kernel: the same bits
-    as a separate compute_logp call, alone and together with the filtered-distribution log-probability."""
+    """sample(..., return_policy_logprob=True): the drawn token's log-probability under the unfiltered softmax comes
+    out of the sampling kernel itself.  Same ids as without it; the value is compute_logp's to 1e-5 (another fixed
+    summation order) and the oracle's to 1e-4, on every route (short top-k, block-wide top-k, dense histogram, radix,
+    fp32 rows, unaligned rows, a masked vocabulary), alone and together with the filtered log-probability."""
+    from oracle import logprob_ref
+    from rl_engine.kernels import _hip
+
     g = torch.Generator().manual_seed(81)
-    for dtype in (torch.bfloat16, torch.float32):
-        logits = (torch.randn(40, 9000, generator=g) * 3).to(dtype).cuda()
+    cases = [dict(top_k=50, top_p=0.9, temperature=0.7), dict(top_k=200, temperature=1.3), dict(top_k=700, top_p=0.95),
+             dict(top_p=0.9, temperature=0.7), dict(top_p=0.9), dict(), dict(top_k=3000, top_p=0.9)]
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        host = (torch.randn(40, 9000, generator=g) * 3).to(dtype)
+        host[5, 4000:] = float("-inf")                                   # masked tail
+        host[6, ::3] = 7.0                                               # 3,000-way tie at the top
+        logits = host.cuda()
         u = torch.rand(40, generator=g).cuda()
-        ids, policy = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
-        assert torch.equal(ids, sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u))
-        assert torch.equal(policy, sampler.compute_logp(logits, ids))
+        for kw in cases:
+            for flags in (0, _hip.SAMPLE_FLAG_BLOCK_WIDE_TOPK, _hip.SAMPLE_FLAG_GENERAL_PATH):
+                ids, policy = sampler.sample(logits, uniforms=u, return_policy_logprob=True, route_flags=flags, **kw)
+                assert torch.equal(ids, sampler.sample(logits, uniforms=u, **kw)), (dtype, kw, flags)
+                assert (policy - sampler.compute_logp(logits, ids)).abs().max().item() <= 1e-5, (dtype, kw, flags)
+                assert (policy.cpu() - logprob_ref.logprob_ref(host, ids.cpu())).abs().max().item() <= 1e-4
         ids2, lp, policy2 = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_logprob=True,
                                            return_policy_logprob=True)
-        assert torch.equal(ids2, ids) and torch.equal(policy2, policy) and (lp <= 0).all()
+        ids1, policy1 = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+        assert torch.equal(ids2, ids1) and torch.equal(policy2, policy1) and (lp <= 0).all()
         # without a temperature the filters only remove mass: the drawn token's filtered probability is at least its policy one
         _, lp1, pol1 = sampler.sample(logits, top_k=50, top_p=0.9, uniforms=u, return_logprob=True, return_policy_logprob=True)
         assert (lp1 >= pol1 - 1e-5).all()
+        # an unaligned view (scalar loads) and a batch split give the same values
+        view = logits[:, 3:8000]
+        a_ids, a_pol = sampler.sample(view, top_k=50, uniforms=u, return_policy_logprob=True)
+        assert (a_pol - sampler.compute_logp(view, a_ids)).abs().max().item() <= 1e-5
+        parts = [sampler.sample(logits[s0:s0 + 10], top_k=50, top_p=0.9, temperature=0.7, uniforms=u[s0:s0 + 10],
+                                return_policy_logprob=True)[1] for s0 in range(0, 40, 10)]
+        assert torch.equal(torch.cat(parts), policy1)
     e_ids, e_pol = sampler.sample(torch.empty(0, 100, dtype=torch.bfloat16, device="cuda"), return_policy_logprob=True)
     assert e_ids.numel() == 0 and e_pol.numel() == 0
