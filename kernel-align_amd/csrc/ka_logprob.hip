@@ -28,6 +28,10 @@ struct RowState {
 
 template <int N, bool ENTROPY>
 __device__ __forceinline__ void fold(RowState &st, const float (&x)[N]) {
+    // No implicit contraction here: fused into an FMA against the fresh product, (st.ml2 - mn * log2e) would return the
+    // rounding residue of a 1e30-sized product instead of 0 while the maximum still sits at the floor (a row that starts
+    // with -inf entries), and 2^residue overflows.  The FMAs below are written out.
+#pragma clang fp contract(off)
     float mn = st.m;
 #pragma unroll
     for (int j = 0; j < N; ++j) mn = fmaxf(mn, x[j]);

@@ -204,3 +204,32 @@ def test_full_size_grpo_group(sampler):
     assert (got_spike[on_spike] > -lse_minus_c - 0.5).all() and (got_spike[on_spike] <= 0).all()
     # every row is a proper log-probability; spike rows that target their spike are ~0
     assert torch.isfinite(flat).all() and (flat <= 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rows_that_start_with_masked_entries(sampler, dtype):
+    """A masked prefix (the first entries of the row are -inf) leaves lanes whose first groups hold nothing but -inf:
+    their running maximum stays at its floor for a while, and the rescale factor between two equal floors must be
+    exactly 1 (an FMA contraction there would return the rounding residue of a 1e30-sized product).  Compared with
+    the oracle, for logprob, entropy and the gradient."""
+    g = torch.Generator().manual_seed(29)
+    logits = (torch.randn(12, 128256, generator=g) * 3).to(dtype)
+    logits[0, :70000] = -math.inf
+    logits[1, :1000] = -math.inf
+    logits[2, 1::2] = -math.inf                      # every other entry
+    logits[3, :] = -math.inf
+    logits[3, 128255] = 1.0                          # a single finite entry at the very end
+    ids = torch.randint(70000, 128256, (12,), generator=g)
+    ids[2] = 2 * (ids[2] // 2)
+    ids[3] = 128255
+    got = sampler.compute_logp(logits.cuda(), ids.cuda()).cpu()
+    assert torch.isfinite(got).all()
+    assert (got.double() - O.logprob_f64(logits, ids)).abs().max().item() <= 2e-5
+    assert abs(got[3].item()) <= 1e-6                # a single finite entry: probability 1
+    lp, ent = sampler.compute_logp_entropy(logits.cuda(), ids.cuda())
+    assert torch.equal(lp.cpu(), got) and (ent.cpu().double() - O.entropy_f64(logits)).abs().max().item() <= TOL
+    grad = torch.randn(12, generator=g)
+    d = sampler.compute_logp_backward(logits.cuda(), ids.cuda(), lp, grad.cuda()).cpu().double()
+    want = O.logprob_backward_closed_form(logits, ids, grad)
+    rel = 2.0 ** -8 if dtype == torch.bfloat16 else 1e-5
+    assert ((d - want).abs() <= rel * want.abs() + 1e-6).all()
