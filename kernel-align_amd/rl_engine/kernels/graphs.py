@@ -1,13 +1,13 @@
 """A decode step of a rollout captured in a HIP graph.
 
-A decode step is two operator calls (sample, then the drawn token's log-probability under the unfiltered
-distribution, which a GRPO ratio is built from).  Both operators only launch kernels on the current stream - no
+A decode step is one operator call: the sampling kernel returns the token and its log-probability under the unfiltered
+distribution (what a GRPO ratio is built from).  The operators only launch kernels on the current stream - no
 allocation inside the library, no memset, no host synchronisation - so the step can be recorded once and replayed,
 alone or as part of a larger capture (the model's forward pass in front of it).
-Measured on an MI355X with ROCm 7.2 (bf16, 128,256 entries, top_k 50 + top_p 0.9): replaying this two-kernel graph on
-its own costs 26 us per step at 64 rows against 22 us for the two eager calls (a graph launch costs more here than
-two kernel launches), so on its own it buys nothing; its use is inside a capture that holds more work, and the test of
-it shows that the operators can be captured at all.
+Measured on an MI355X with ROCm 7.2 (bf16, 128,256 entries, top_k 50 + top_p 0.9): replaying this graph on its own
+costs 21 us per step at 64 rows against 16 us for the eager call (a graph launch costs more here than a kernel
+launch), so on its own it buys nothing; its use is inside a capture that holds more work, and the test of it shows
+that the operators can be captured at all.
 
     step = GraphedDecodeStep(sampler, batch=64, vocab=128256, top_k=50, top_p=0.9, temperature=0.7)
     step.logits.copy_(next_logits)          # or let the model write into step.logits
