@@ -127,6 +127,16 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
         torch.cuda.synchronize()
         kernel_ms = ev0.elapsed_time(ev1) / 200
         out[f"kernel_ms_b{batch}"] = kernel_ms
+        # a decode step: the id and its log-probability under the unfiltered softmax from the one kernel
+        for _ in range(5):
+            sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(100):
+            sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+        ev1.record()
+        torch.cuda.synchronize()
+        out[f"decode_step_ms_b{batch}"] = ev0.elapsed_time(ev1) / 100
         if batch == 256:
             gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
