@@ -24,13 +24,6 @@
 
 #include "ka_common.h"
 
-// Timing experiments only (results are wrong with any LM_ABL_* switch set).
-#ifdef LM_ABL_HOTCOPY
-#define LM_HOT(x_) ((x_) & 1)
-#else
-#define LM_HOT(x_) (x_)
-#endif
-
 namespace ka {
 namespace {
 
@@ -46,59 +39,29 @@ constexpr int LM_THREADS = 256;
 // V = 128,256 (501 tiles, 64 splits of 7 or 8) 64 rows take 0.74 ms, against 5.3 ms with 63 tiles per split.
 constexpr int LM_TILES_PER_SPLIT = 8;
 // Group (of 32 per slab) at which the next slab is waited for.  It lies in the last k-step: the first fragments of
-// the next slab are loaded into the buffer that the k-steps 0 and 2 read, right behind the barrier.  28 measures 2 %
-// slower.
-#ifndef LM_BAR_GROUP
-#define LM_BAR_GROUP 24
-#endif
-constexpr int LM_BAR = LM_BAR_GROUP;
-static_assert(LM_BAR >= 24 && LM_BAR <= 28, "the barrier group must lie in the last k-step and leave four groups for the reads");
+// the next slab are loaded into the buffer that the k-steps 0 and 2 read, right behind the barrier.  (28 measures 2 %
+// slower.)
+constexpr int LM_BAR = 24;
 // When the sixteen copies of a slab are requested.  A slab's window opens behind the barrier that frees its stage
-// (group LM_BAR of the slab two before it) and closes at the next barrier, 32 groups later; position p of the window
-// is group (LM_BAR + p) % 32.  lm_copy_pos(c) is the position of copy c (non-decreasing in c, copies complete in
-// order).  One copy per group over the first 16 positions keeps the vector memory path of the CU busy without a
-// gap for half of every slab and idle for the other half; the schedules below spread them.
-#ifndef LM_COPY_SCHEDULE
-#define LM_COPY_SCHEDULE 0
-#endif
-__host__ __device__ constexpr int lm_copy_pos(int c) {
-    return LM_COPY_SCHEDULE == 0 ? c                                  // positions 0..15
-         : LM_COPY_SCHEDULE == 1 ? (c < 8 ? c : 8 + 2 * (c - 8))      // 0..7, then every other group up to 22
-         : LM_COPY_SCHEDULE == 2 ? (3 * c) / 2                        // two per three groups: 0,1,3,4,...,22
-         : LM_COPY_SCHEDULE == 3 ? (c < 4 ? c : 4 + (3 * (c - 4)) / 2) // 0..3, then two per three up to 21
-         : LM_COPY_SCHEDULE == 4 ? c / 2                              // two per group: 0..7
-         : LM_COPY_SCHEDULE == 6 ? (c < 8 ? c : c + 4)                 // 0..7, then 12..19
-         : LM_COPY_SCHEDULE == 7 ? (c < 8 ? c : c + 2)                 // 0..7, then 10..17
-         : LM_COPY_SCHEDULE == 8 ? (c < 8 ? c : c - 4)                 // 0..7, and the second eight doubled up on 4..11
-         : (5 * c) / 4;                                               // four per five groups: 0..18
-}
-__host__ __device__ constexpr int lm_copies_before(int pos) {  // copies with a position below pos
-    int n = 0;
-    for (int c = 0; c < 16; ++c) n += lm_copy_pos(c) < pos ? 1 : 0;
-    return n;
-}
-__host__ __device__ constexpr int lm_copy_at(int pos, int k) {  // k-th copy requested at position pos, -1: none
-    for (int c = 0; c < 16; ++c)
-        if (lm_copy_pos(c) == pos && k-- == 0) return c;
-    return -1;
-}
-struct CopyTable {  // [group][k]: the copies requested in a group, -1 = none (a table: the group loop must stay cheap to unroll)
-    signed char at[32][2];
+// (group LM_BAR of the slab two before it) and closes at the next barrier, 32 groups later; copy c is requested at
+// position c of the window, i.e. in group (LM_BAR + c) % 32: one copy per group over the first half of the window
+// (spreading them over the whole window, or two per group, measured slower).
+struct CopyTable {  // [group]: the copy requested in that group, -1 = none (a table: the group loop must stay cheap to unroll)
+    signed char at[32];
     constexpr CopyTable() : at{} {
-        for (int g = 0; g < 32; ++g)
-            for (int k = 0; k < 2; ++k) at[g][k] = (signed char)lm_copy_at(g >= LM_BAR ? g - LM_BAR : g + 32 - LM_BAR, k);
+        for (int g = 0; g < 32; ++g) {
+            const int pos = g >= LM_BAR ? g - LM_BAR : g + 32 - LM_BAR;
+            at[g] = (signed char)(pos < 16 ? pos : -1);
+        }
     }
 };
 constexpr CopyTable kCopyTable{};
-constexpr int LM_FIRST = lm_copies_before(32 - LM_BAR);
-// Group in which the copy cursor moves on to the next slab: anywhere between the last copy of a window and the first
-// of the next one.
-#ifndef LM_ADV_GROUP
-#define LM_ADV_GROUP 12
-#endif
-constexpr int LM_ADV = LM_ADV_GROUP;
-static_assert(LM_ADV <= LM_BAR && LM_ADV + 32 - LM_BAR > lm_copy_pos(15), "the cursor moves between two windows");  // copies requested in the groups LM_BAR .. 31
-static_assert(lm_copy_pos(15) <= 23, "the last copy needs a few groups to land before the barrier");
+constexpr int LM_FIRST = 32 - LM_BAR;  // copies of a slab requested before the slab boundary (groups LM_BAR .. 31)
+// Group in which the copy cursor moves on to the next slab: between the last copy of a window and the first of the
+// next one.
+constexpr int LM_ADV = 12;
+static_assert(LM_BAR >= 24 && LM_BAR <= 28, "the barrier group must lie in the last k-step and leave four groups for the reads");
+static_assert(LM_ADV <= LM_BAR && LM_ADV + 32 - LM_BAR > 15, "the cursor moves between two windows");
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr double kLn2 = 0.693147180559945309417232;
 constexpr float kFloor = -1.0e30f;
@@ -212,9 +175,6 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // A workgroup walks its items v = blockIdx.x, + gridDim.x, ...: with one workgroup per CU nothing is
     // dispatched between items, and the copies of an item's first slabs are requested while the item before
     // it is still being multiplied.
-#ifdef LM_ABL_CLOCK
-    const uint64_t clk0 = __builtin_readcyclecounter(), rt0 = __builtin_amdgcn_s_memrealtime();
-#endif
     const ItemOrder order(n_token_blocks, n_splits);
     const int stride = gridDim.x;
     const int nk = hdim / LM_BK;
@@ -251,12 +211,12 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     do {                                                                                                     \
         if constexpr (!WIDE) {                                                                               \
             _Pragma("unroll") for (int j = 0; j < 8; ++j)                                                    \
-                woff[j] = uint32_t(min(LM_HOT(vt_) * LM_BM + cp_row + 32 * j, vocab - 1)) * row_bytes + cp_chunk[j] * 16u; \
+                woff[j] = uint32_t(min(vt_ * LM_BM + cp_row + 32 * j, vocab - 1)) * row_bytes + cp_chunk[j] * 16u; \
         }                                                                                                    \
     } while (0)
     const uint32_t row_bytes = uint32_t(hdim) * 2u;
     const char *hbase = reinterpret_cast<const char *>(hidden);  // WIDE: first hidden row of the cursor's token block
-    LM_SET_HOFF(LM_HOT(tb) * LM_BN);
+    LM_SET_HOFF(tb * LM_BN);
     const int wave_lds = __builtin_amdgcn_readfirstlane(wave) * 512;  // bf16 elements: 8 rows of 64
     const char *const wbytes = reinterpret_cast<const char *>(weight);
 
@@ -264,12 +224,9 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // rows.  W first, because its copies take longer (a W tile is streamed once per pass, the hidden rows of the
     // token block come back from cache at every tile) and the first copies of a window have the longest time to
     // land: measured 5 % faster than alternating W and hidden copies, 4 % faster than hidden first.
-#ifdef LM_ABL_NOCOPY
-#define LM_ISSUE_ONE(c_, vt_, kt_, stage_) do { } while (0)
-#else
 #define LM_ISSUE_ONE(c_, vt_, kt_, stage_)                                                                   \
     do {                                                                                                     \
-        const size_t kb_ = LM_HOT(size_t(kt_)) * (LM_BK * 2);                                                \
+        const size_t kb_ = size_t(kt_) * (LM_BK * 2);                                                \
         uint16_t *sa_ = lds + (stage_) * LM_STAGE_ELEMS + wave_lds + ((c_) & 7) * 2048;                        \
         if ((c_) < 8) {                                                                                      \
             if constexpr (WIDE) {                                                                            \
@@ -283,7 +240,6 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             __builtin_amdgcn_global_load_lds(hbase + kb_ + hoff[(c_) & 7], (lds_void *)(sa_ + LM_BM * LM_BK), 16, 0, 0); \
         }                                                                                                    \
     } while (0)
-#endif
 
     // Copy cursor: the next slab to request.  It runs up to two slabs ahead of the MFMAs and crosses from an
     // item's last slab into the first slab of the workgroup's next item.  Past the last slab of the last item
@@ -304,7 +260,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                 vt_c = lm_split_begin(sp_, n_vtiles, n_splits);                                              \
                 vt_end_c = lm_split_begin(sp_ + 1, n_vtiles, n_splits);                                      \
                 kt_c = 0;                                                                                    \
-                LM_SET_HOFF(LM_HOT(tb_) * LM_BN);                                                                    \
+                LM_SET_HOFF(tb_ * LM_BN);                                                                    \
                 LM_SET_WOFF(vt_c);                                                                           \
             }                                                                                                \
         }                                                                                                    \
@@ -389,23 +345,15 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][tm], fb[kk & 1][tn], acc[tm][tn], 0, 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-#ifndef LM_ABL_NOREAD
                 if (kk < 3 && sub < 4) {  // both reads early in the k-step: they have returned when it ends
                     fa[(kk + 1) & 1][sub] = LM_FRAG(pa[kk + 1], sub);
                     fb[(kk + 1) & 1][sub] = LM_FRAG(pb[kk + 1], sub);
                 }
-#endif
                 if (g == LM_BAR) {
                     // Builtins rather than inline asm: the compiler's own wait-count bookkeeping sees them, so it
                     // does not add a conservative lgkmcnt(0) behind the fresh reads that follow.
-#ifdef LM_ABL_NOVMWAIT
-                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only
-#else
                     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-#endif
-#ifndef LM_ABL_NOBAR
                     __builtin_amdgcn_s_barrier();
-#endif
                     // every read of this slab has been issued: the pointers move to the stage of the next slab
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
@@ -414,12 +362,10 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                     }
                     stage_step = -stage_step;
                 }
-#ifndef LM_ABL_NOREAD
                 if (g >= LM_BAR && g < LM_BAR + 4) {
                     fa[0][g - LM_BAR] = LM_FRAG(pa[0], g - LM_BAR);
                     fb[0][g - LM_BAR] = LM_FRAG(pb[0], g - LM_BAR);
                 }
-#endif
                 __builtin_amdgcn_sched_barrier(0);
                 {
                     const int m = sub * 2 + 1, tm = m >> 2, tn = m & 3;
@@ -430,9 +376,8 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                     // copies of this group: behind the barrier they belong to the slab whose window has just opened
                     // (the cursor has moved on to it) and go to the stage that the barrier has freed
                     if (g == LM_ADV) LM_ADVANCE_COPY_CURSOR();
-                    const int c0 = kCopyTable.at[g][0], c1 = kCopyTable.at[g][1];  // compile-time: g is unrolled
+                    const int c0 = kCopyTable.at[g];  // compile-time: g is unrolled
                     if (c0 >= 0) LM_ISSUE_ONE(c0, vt_c, kt_c, g >= LM_BAR ? stage : stage ^ 1);
-                    if (c1 >= 0) LM_ISSUE_ONE(c1, vt_c, kt_c, g >= LM_BAR ? stage : stage ^ 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -443,12 +388,6 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         // Vocabulary row of acc[tm][tn][r]: vrow0 + tm*32 + (r/4)*8 + r%4.
         const int vrow0 = vt * LM_BM + wave_m * 128 + lhalf * 4;
         const int limit = vocab - vrow0;  // rows at offset >= limit lie past the vocabulary (last tile only)
-#ifdef LM_ABL_NOEPI
-#pragma unroll
-        for (int tn = 0; tn < 4; ++tn)
-            m_run[tn] = fmaxf(m_run[tn], (acc[0][tn][0] + acc[1][tn][1]) + (acc[2][tn][2] + acc[3][tn][3]));
-        if (false)
-#endif
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
             // keep the four token blocks apart: only 64 accumulators are live in VGPRs at a time
@@ -594,12 +533,6 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     if (v >= n_virtual) break;
     }  // items
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the trailing (redundant) slab copies still write LDS
-#ifdef LM_ABL_CLOCK
-    if (blockIdx.x == 0 && tid == 0) {  // shader cycles per 100 MHz tick over the life of this workgroup
-        const uint64_t clk1 = __builtin_readcyclecounter(), rt1 = __builtin_amdgcn_s_memrealtime();
-        partials[0].pad = float(double(clk1 - clk0) / double(rt1 - rt0));
-    }
-#endif
 }
 
 __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict__ partials,
