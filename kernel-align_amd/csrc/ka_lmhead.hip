@@ -15,10 +15,13 @@
 //     after each vocabulary tile is register-local, with no cross-lane traffic;
 //   * each wavefront computes 128 vocab x 128 tokens = 4 x 4 MFMA blocks
 //     (256 fp32 accumulators per lane);
-//   * the vocabulary is cut into fixed splits of LM_TILES_PER_SPLIT tiles (a
-//     function of the vocabulary only, so results do not depend on the number of
-//     rows); every (token block, split) writes one (max, sum, target logit)
-//     partial per token and a second kernel folds the partials in split order.
+//   * the vocabulary is cut into fixed splits of at most LM_TILES_PER_SPLIT tiles and every split into LM_SUBS
+//     units of at most two tiles (a function of the vocabulary only).  A row's result is defined as: per unit an
+//     online (max, sum, target logit), the units of a split folded in order, the splits folded in order - so it
+//     does not depend on the number of rows, nor on who folds: with many rows an item is a (token block, split)
+//     pair and the kernel folds the units itself; with few rows (fewer items than CUs) an item is a
+//     (token block, unit) pair, so that one token block occupies every CU, and the second kernel folds the
+//     units with the same operations.  Same bits either way.
 // Logits stay in fp32 (the accumulators are not rounded to bf16).
 #include <mutex>
 
@@ -32,12 +35,16 @@ constexpr int LM_BN = 256;      // tokens per workgroup
 constexpr int LM_BK = 64;       // hidden slab: one 128-byte line per row
 constexpr int LM_STAGES = 2;    // LDS: the slab in use and the slab in flight
 constexpr int LM_STAGE_ELEMS = (LM_BM + LM_BN) * LM_BK;  // bf16 elements per LDS stage (64 KB)
-constexpr int LM_XCH_BYTES = 2 * 4 * 32 * 4 * 4;  // exchange area of the end-of-item fold: [wave_n][tn][32 lanes][4 floats]
-constexpr int LM_LDS_BYTES = LM_STAGES * LM_STAGE_ELEMS * 2 + LM_XCH_BYTES;
+constexpr int LM_XCH_BYTES = 2 * 4 * 32 * 4 * 4;  // exchange area of the end-of-unit fold: [wave_n][tn][32 lanes][4 floats]
+constexpr int LM_SPLIT_ACC_BYTES = LM_XCH_BYTES;  // running partial of the item's split, same shape (touched by its own lane only)
+constexpr int LM_LDS_BYTES = LM_STAGES * LM_STAGE_ELEMS * 2 + LM_XCH_BYTES + LM_SPLIT_ACC_BYTES;
 constexpr int LM_THREADS = 256;
 // Vocabulary tiles per split (at most).  Short splits let a single token block occupy many CUs: at
 // V = 128,256 (501 tiles, 64 splits of 7 or 8) 64 rows take 0.74 ms, against 5.3 ms with 63 tiles per split.
 constexpr int LM_TILES_PER_SPLIT = 8;
+// Units per split.  With 8-tile splits a unit is two tiles: at V = 128,256 a single token block then makes 256 items,
+// one per CU, of 1 - 2 tiles each (64 rows: 0.73 ms with whole splits as items).
+constexpr int LM_SUBS = 4;
 // Group (of 32 per slab) at which the next slab is waited for.  It lies in the last k-step: the first fragments of
 // the next slab are loaded into the buffer that the k-steps 0 and 2 read, right behind the barrier.  (28 measures 2 %
 // slower.)
@@ -74,12 +81,41 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 __host__ __device__ inline int lm_n_splits(int n_vtiles) {
     return n_vtiles <= 8 ? n_vtiles : 8 * ((n_vtiles + 8 * LM_TILES_PER_SPLIT - 1) / (8 * LM_TILES_PER_SPLIT));
 }
-// First vocabulary tile of split sp (sp == n_splits: the end).
-__host__ __device__ inline int lm_split_begin(int sp, int n_vtiles, int n_splits) {
-    return int(uint64_t(sp) * uint64_t(n_vtiles) / uint64_t(n_splits));
+// The plan in the form the kernels use (no division on the device): every split holds `base` tiles, the first `rem`
+// splits one more.
+struct SplitPlan {
+    int n_vtiles, n_splits, base, rem;
+    __host__ __device__ SplitPlan(int n_vtiles_, int n_splits_)
+        : n_vtiles(n_vtiles_), n_splits(n_splits_), base(n_vtiles_ / n_splits_), rem(n_vtiles_ % n_splits_) {}
+    // First vocabulary tile of split sp (sp == n_splits: the end).
+    __host__ __device__ int split_begin(int sp) const { return sp * base + (sp < rem ? sp : rem); }
+    // First vocabulary tile of unit u = split * LM_SUBS + j (u == n_splits * LM_SUBS: the end).  Units of a split
+    // shorter than LM_SUBS tiles may be empty.
+    __host__ __device__ int unit_begin(int u) const {
+        const int sp = u / LM_SUBS, j = u % LM_SUBS;
+        const int len = sp < n_splits ? base + (sp < rem ? 1 : 0) : 0;
+        return split_begin(sp) + j * len / LM_SUBS;
+    }
+};
+
+// Fold of two partial results of one row, (M, S, X, A) <- (M, S, X, A) + (m, s, x, a): the operation by which the units
+// of a split are combined, in unit order, starting from (kFloorM, 0, -inf, 0).  Written out operation by operation
+// and never contracted, because two kernels must produce the same bits with it.
+__device__ __forceinline__ void lm_fold_unit(float &M, float &S, float &X, float &A, float m, float s, float x, float a) {
+#pragma clang fp contract(off)
+    const float mn = fmaxf(M, m);
+    const float f_old = fast_exp2((M - mn) * 1.44269504088896340736f);
+    const float f_new = fast_exp2((m - mn) * 1.44269504088896340736f);
+    const float s_old = S * f_old, s_new = s * f_new;
+    const float a_old = A * f_old, a_new = a * f_new;
+    S = s_old + s_new;
+    A = a_old + a_new;
+    X = fmaxf(X, x);
+    M = mn;
 }
 
-// Work items are (token block, split) pairs, grouped into super-tiles of tbw token blocks x 32 / tbw splits.  Item v
+// Work items are (token block, split) pairs - or, with few rows, (token block, unit) pairs, for which "split" below
+// reads "unit" - grouped into super-tiles of tbw token blocks x 32 / tbw splits.  Item v
 // belongs to the workgroup v % grid; with a grid of 256 that workgroup sits on XCD v % 8 and holds position
 // (v / 8) % 32 of the super-tile that its XCD works on in round v / 256, so the 32 CUs of an XCD run one
 // super-tile side by side and fetch 12 distinct slabs per step instead of 64.
@@ -93,26 +129,45 @@ __host__ __device__ inline int lm_split_begin(int sp, int n_vtiles, int n_splits
 // blocks or more: every XCD then passes over W half as often; 2 - 3 % faster at 32,768 rows), else 4 x 8.
 // Neither the order nor the shape changes any result.  Pairs past the ends of the two ranges are not items.
 struct ItemOrder {
+    int fine;       // 1: items are (token block, unit) pairs in the plain order described below
+    int n_token_blocks, n_cols;  // the two ranges (n_cols: splits, or units)
+    SplitPlan plan;
     int tbw, spw;   // token blocks and splits of a super-tile (tbw * spw == 32)
     int sp_groups;  // ceil(n_splits / spw)
     int full;       // token-block groups handled eight at a time
     int rest;       // token-block groups left over (0..7)
-    __host__ __device__ ItemOrder(int n_token_blocks, int n_splits) {
+    __host__ __device__ ItemOrder(int n_token_blocks_, const SplitPlan &plan_, int fine_) : plan(plan_) {
+        fine = fine_;
+        n_token_blocks = n_token_blocks_;
+        n_cols = fine ? plan.n_splits * LM_SUBS : plan.n_splits;
         tbw = n_token_blocks >= 64 ? 8 : 4;
         spw = 32 / tbw;
         const int tb_groups = (n_token_blocks + tbw - 1) / tbw;
-        sp_groups = (n_splits + spw - 1) / spw;
+        sp_groups = (n_cols + spw - 1) / spw;
         full = tb_groups / 8 * 8;
         rest = tb_groups - full;
     }
     __host__ __device__ int rounds_full() const { return full / 8 * sp_groups; }
-    __host__ __device__ int64_t n_virtual() const {  // item indices in use: 256 per round
-        return (int64_t(rounds_full()) + (rest * sp_groups + 7) / 8) * 256;
+    __host__ __device__ int64_t n_virtual() const {  // item indices in use
+        if (fine) return int64_t(n_token_blocks) * ((n_cols + 7) / 8 * 8);
+        return (int64_t(rounds_full()) + (rest * sp_groups + 7) / 8) * 256;  // 256 per round
+    }
+    // Vocabulary tiles [begin, end) of column c.
+    __host__ __device__ int col_begin(int c) const {
+        return fine ? plan.unit_begin(c) : plan.split_begin(c);
     }
 };
 
-__device__ __forceinline__ bool lm_decode(int v, const ItemOrder &order, int n_token_blocks, int n_splits, int &tb,
-                                          int &sp) {
+// Few rows: item v = ((unit / 8) * n_token_blocks + token block) * 8 + unit % 8, so that unit u is worked on by XCD
+// u % 8 for all token blocks at about the same time (its W tiles are fetched from HBM once) and consecutive units
+// go to different XCDs.  Empty units are not items.
+__device__ __forceinline__ bool lm_decode(int v, const ItemOrder &order, int &tb, int &sp) {
+    if (order.fine) {
+        const int q = v / 8;
+        tb = q % order.n_token_blocks;
+        sp = (q / order.n_token_blocks) * 8 + v % 8;
+        return sp < order.n_cols && order.col_begin(sp) < order.col_begin(sp + 1);
+    }
     const int xcd = v % 8, slot = v / 8;
     const int round = slot / 32, w = slot % 32;
     int tg, sg;
@@ -127,14 +182,13 @@ __device__ __forceinline__ bool lm_decode(int v, const ItemOrder &order, int n_t
     }
     tb = tg * order.tbw + w / order.spw;
     sp = sg * order.spw + w % order.spw;
-    return tb < n_token_blocks && sp < n_splits;
+    return tb < order.n_token_blocks && sp < order.n_cols;
 }
 // The next item of the workgroup that holds item v: indices advance by the grid size.  >= n_virtual: none.
-__device__ __forceinline__ int lm_next_item(int v, int stride, int n_virtual, const ItemOrder &order,
-                                            int n_token_blocks, int n_splits) {
+__device__ __forceinline__ int lm_next_item(int v, int stride, int n_virtual, const ItemOrder &order) {
     int tb, sp;
     do v += stride;
-    while (v < n_virtual && !lm_decode(v, order, n_token_blocks, n_splits, tb, sp));
+    while (v < n_virtual && !lm_decode(v, order, tb, sp));
     return v;
 }
 
@@ -160,8 +214,8 @@ typedef __attribute__((address_space(3))) void lds_void;
 template <bool WIDE, bool ENTROPY>
 __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
-    Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_splits, int n_token_blocks,
-    int n_vtiles, int n_virtual) {
+    Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_token_blocks,
+    SplitPlan plan, int n_virtual, int fine) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [stage][A = W slab | B = hidden slab]
 
     const int tid = threadIdx.x;
@@ -175,12 +229,11 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // A workgroup walks its items v = blockIdx.x, + gridDim.x, ...: with one workgroup per CU nothing is
     // dispatched between items, and the copies of an item's first slabs are requested while the item before
     // it is still being multiplied.
-    const ItemOrder order(n_token_blocks, n_splits);
+    const ItemOrder order(n_token_blocks, plan, fine);
     const int stride = gridDim.x;
     const int nk = hdim / LM_BK;
-    int v = blockIdx.x, tb, sp;
-    if (!lm_decode(v, order, n_token_blocks, n_splits, tb, sp))
-        v = lm_next_item(v, stride, n_virtual, order, n_token_blocks, n_splits);
+    int v = blockIdx.x, tb, sp;  // sp: the item's column (split, or unit when fine)
+    if (!lm_decode(v, order, tb, sp)) v = lm_next_item(v, stride, n_virtual, order);
     if (v >= n_virtual) return;
 
     float m_run[4], ml2_run[4], s_run[4], xt[4];  // ml2_run = m_run * log2(e), kept so that it is never recomputed
@@ -244,26 +297,37 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // Copy cursor: the next slab to request.  It runs up to two slabs ahead of the MFMAs and crosses from an
     // item's last slab into the first slab of the workgroup's next item.  Past the last slab of the last item
     // it stays there (redundant copies into the idle stage), so that every step issues the same copies.
-    int v_c = v, vt_c = lm_split_begin(sp, n_vtiles, n_splits), vt_end_c = lm_split_begin(sp + 1, n_vtiles, n_splits);
+    int v_c = v, vt_c = order.col_begin(sp), vt_end_c = order.col_begin(sp + 1);
     int kt_c = 0;
     LM_SET_WOFF(vt_c);
-#define LM_ADVANCE_COPY_CURSOR()                                                                              \
+    // The cursor moves once per slab.  Where to is worked out ahead of the slab's unrolled groups (scalar work, with a
+    // search for the workgroup's next item at the end of an item: too long to sit inside the unrolled loop) and
+    // committed in group LM_ADV.
+    int nx_v = v, nx_vt = vt_c, nx_vt_end = vt_end_c, nx_kt = 0, nx_tb = -1;  // nx_tb >= 0: the token block changes
+#define LM_PLAN_CURSOR_MOVE()                                                                                 \
     do {                                                                                                     \
-        if (kt_c + 1 < nk) ++kt_c;                                                                           \
-        else if (vt_c + 1 < vt_end_c) { ++vt_c; kt_c = 0; LM_SET_WOFF(vt_c); }                                \
+        nx_v = v_c; nx_vt = vt_c; nx_vt_end = vt_end_c; nx_kt = kt_c; nx_tb = -1;                            \
+        if (kt_c + 1 < nk) nx_kt = kt_c + 1;                                                                 \
+        else if (vt_c + 1 < vt_end_c) { nx_vt = vt_c + 1; nx_kt = 0; }                                       \
         else {                                                                                               \
-            const int nv_ = lm_next_item(v_c, stride, n_virtual, order, n_token_blocks, n_splits);       \
+            const int nv_ = lm_next_item(v_c, stride, n_virtual, order);                                     \
             if (nv_ < n_virtual) {                                                                           \
                 int tb_, sp_;                                                                                \
-                lm_decode(nv_, order, n_token_blocks, n_splits, tb_, sp_);                               \
-                v_c = nv_;                                                                                   \
-                vt_c = lm_split_begin(sp_, n_vtiles, n_splits);                                              \
-                vt_end_c = lm_split_begin(sp_ + 1, n_vtiles, n_splits);                                      \
-                kt_c = 0;                                                                                    \
-                LM_SET_HOFF(tb_ * LM_BN);                                                                    \
-                LM_SET_WOFF(vt_c);                                                                           \
+                lm_decode(nv_, order, tb_, sp_);                                                             \
+                nx_v = nv_;                                                                                  \
+                nx_vt = order.col_begin(sp_);                                                                \
+                nx_vt_end = order.col_begin(sp_ + 1);                                                        \
+                nx_kt = 0;                                                                                   \
+                nx_tb = tb_;                                                                                 \
             }                                                                                                \
         }                                                                                                    \
+    } while (0)
+#define LM_COMMIT_CURSOR_MOVE()                                                                               \
+    do {                                                                                                     \
+        const bool new_tile_ = nx_vt != vt_c || nx_tb >= 0;                                                  \
+        v_c = nx_v; vt_c = nx_vt; vt_end_c = nx_vt_end; kt_c = nx_kt;                                        \
+        if (nx_tb >= 0) LM_SET_HOFF(nx_tb * LM_BN);                                                          \
+        if (new_tile_) LM_SET_WOFF(vt_c);                                                                    \
     } while (0)
     // Fragment addresses.  swz() of a fragment row does not depend on the 32-row block (t * 32 and wave * 128 do not
     // touch bits 1..3), so block t of an operand sits t * 4096 bytes behind block 0 and only the k-step changes the
@@ -294,7 +358,8 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     // program order would issue too late to hide its latency: the order below is pinned with sched_barrier.
 #pragma unroll
     for (int c = 0; c < 16; ++c) LM_ISSUE_ONE(c, vt_c, kt_c, 0);
-    LM_ADVANCE_COPY_CURSOR();
+    LM_PLAN_CURSOR_MOVE();
+    LM_COMMIT_CURSOR_MOVE();
 #pragma unroll
     for (int c = 0; c < LM_FIRST; ++c) LM_ISSUE_ONE(c, vt_c, kt_c, 1);  // the rest of slab 1 follows in the groups of slab 0
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LM_FIRST) : "memory");  // copies complete in order: slab 0 is in
@@ -306,12 +371,33 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     }
 
     int stage = 0;
+    float *const xch = reinterpret_cast<float *>(lds + LM_STAGES * LM_STAGE_ELEMS);  // [wave_n][tn][32][4]
+    float *const split_acc = xch + LM_XCH_BYTES / 4;                                  // same shape
+    const bool folder = wave_m == 0 && lhalf == 0;  // the lanes that end up with a token's folded partial
     for (;;) {  // items of this workgroup; v is a valid item here
-    lm_decode(v, order, n_token_blocks, n_splits, tb, sp);
+    lm_decode(v, order, tb, sp);
     const int tok0 = tb * LM_BN;
-    const int vt_begin = lm_split_begin(sp, n_vtiles, n_splits);
-    const int vt_end = lm_split_begin(sp + 1, n_vtiles, n_splits);
     // This lane's four tokens (one per 32-column block of the wave tile) and their targets.
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+        const int n = tok0 + wave_n * 128 + tn * 32 + l32;
+        int64_t id = -1;
+        if (n < n_rows) id = ids[n];
+        target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
+        if (!fine && folder) {  // the split's running partial starts empty
+            float *p = split_acc + ((wave_n * 4 + tn) * 32 + l32) * 4;
+            p[0] = kFloor;
+            p[1] = 0.0f;
+            p[2] = -__builtin_inff();
+            p[3] = 0.0f;
+        }
+    }
+    // The units of the item: its own when the item is a unit, else those of its split, in order.
+    const int u_first = fine ? sp : sp * LM_SUBS, u_last = fine ? sp + 1 : (sp + 1) * LM_SUBS;
+    for (int u = u_first; u < u_last; ++u) {
+    const int vt_begin = plan.unit_begin(u);
+    const int vt_end = plan.unit_begin(u + 1);
+    if (vt_begin == vt_end) continue;  // (workgroup-uniform) a split of fewer than LM_SUBS tiles has empty units
 #pragma unroll
     for (int tn = 0; tn < 4; ++tn) {
         m_run[tn] = kFloor;
@@ -319,10 +405,6 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         s_run[tn] = 0.0f;
         a_run[tn] = 0.0f;
         xt[tn] = -__builtin_inff();
-        const int n = tok0 + wave_n * 128 + tn * 32 + l32;
-        int64_t id = -1;
-        if (n < n_rows) id = ids[n];
-        target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
     }
     for (int vt = vt_begin; vt < vt_end; ++vt) {
         f32x16 acc[4][4];
@@ -336,6 +418,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         // Per group: first MFMA, the group's fragment reads, second MFMA, the group's copy: each MFMA covers the
         // issue of at most two other instructions.
         for (int kt = 0; kt < nk; ++kt) {
+            LM_PLAN_CURSOR_MOVE();
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int g = 0; g < 32; ++g) {
@@ -375,7 +458,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
                 {
                     // copies of this group: behind the barrier they belong to the slab whose window has just opened
                     // (the cursor has moved on to it) and go to the stage that the barrier has freed
-                    if (g == LM_ADV) LM_ADVANCE_COPY_CURSOR();
+                    if (g == LM_ADV) LM_COMMIT_CURSOR_MOVE();
                     const int c0 = kCopyTable.at[g];  // compile-time: g is unrolled
                     if (c0 >= 0) LM_ISSUE_ONE(c0, vt_c, kt_c, g >= LM_BAR ? stage : stage ^ 1);
                 }
@@ -390,6 +473,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         const int limit = vocab - vrow0;  // rows at offset >= limit lie past the vocabulary (last tile only)
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
+#pragma clang fp contract(off)  // (mn * log2e feeds a difference: as part of an FMA it would not cancel at the floor)
             // keep the four token blocks apart: only 64 accumulators are live in VGPRs at a time
             __builtin_amdgcn_sched_barrier(0);
             const int d = target[tn] - (vt * LM_BM + wave_m * 128);
@@ -492,9 +576,8 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         xt[tn] = fmaxf(xt[tn], ox);
     }
     // ---- fold the two vocabulary halves of the tile through LDS (upper half -> lower half) ----
-    // The exchange area lies behind the two stages, which already receive the first slabs of the next item.
-    // One barrier is enough: the area is written again only after the next item's slabs, each with a barrier.
-    float *xch = reinterpret_cast<float *>(lds + LM_STAGES * LM_STAGE_ELEMS);  // [wave_n][tn][32][4]
+    // The exchange area lies behind the two stages, which already receive the slabs of the next unit or item.
+    // One barrier is enough: the area is written again only after another unit's slabs, each with a barrier.
     if (wave_m == 1 && lhalf == 0) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
@@ -509,7 +592,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only: the slab copies in flight are not waited for
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (wave_m == 0 && lhalf == 0) {
+    if (folder) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
             const float *p = xch + ((wave_n * 4 + tn) * 32 + l32) * 4;
@@ -517,52 +600,135 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             const float mm = fmaxf(m_run[tn], om);
             const float f_own = fast_exp2((m_run[tn] - mm) * kLog2e), f_other = fast_exp2((om - mm) * kLog2e);
             const float s = s_run[tn] * f_own + os * f_other;
+            float a = 0.0f;
+            if constexpr (ENTROPY) a = a_run[tn] * f_own + p[3] * f_other;
+            const float x = fmaxf(xt[tn], ox);
+            const int n = tok0 + wave_n * 128 + tn * 32 + l32;
+            if (fine) {  // the unit's partial goes out as it is; the second kernel folds the units
+                if (n < n_rows) {
+                    Partial out;
+                    out.m = mm;
+                    out.s = s;
+                    out.xt = x;
+                    out.pad = a;
+                    partials[size_t(u) * n_rows + n] = out;
+                }
+            } else {
+                float *q = split_acc + ((wave_n * 4 + tn) * 32 + l32) * 4;
+                float M = q[0], S = q[1], X = q[2], A = q[3];
+                lm_fold_unit(M, S, X, A, mm, s, x, a);
+                q[0] = M;
+                q[1] = S;
+                q[2] = X;
+                q[3] = A;
+            }
+        }
+    }
+    }  // units
+    if (!fine && folder) {
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+            const float *q = split_acc + ((wave_n * 4 + tn) * 32 + l32) * 4;
             const int n = tok0 + wave_n * 128 + tn * 32 + l32;
             if (n < n_rows) {
                 Partial out;
-                out.m = mm;
-                out.s = s;
-                out.xt = fmaxf(xt[tn], ox);
-                out.pad = 0.0f;
-                if constexpr (ENTROPY) out.pad = a_run[tn] * f_own + p[3] * f_other;
+                out.m = q[0];
+                out.s = q[1];
+                out.xt = q[2];
+                out.pad = q[3];
                 partials[size_t(sp) * n_rows + n] = out;
             }
         }
     }
-    v = lm_next_item(v, stride, n_virtual, order, n_token_blocks, n_splits);
+    v = lm_next_item(v, stride, n_virtual, order);
     if (v >= n_virtual) break;
     }  // items
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the trailing (redundant) slab copies still write LDS
 }
 
+// The fold of a row's split partials, in split order, and the two results.  get(sp) returns the partial of split sp.
+// Written out operation by operation (no contraction): whoever produced the split partials, the bits are the same.
+template <typename Get>
+__device__ __forceinline__ void lm_finish_row(Get get, int n_splits, int64_t id, int vocab, float *out_slot, float *entropy_slot) {
+#pragma clang fp contract(off)
+    float mm = kFloor;
+    for (int sp = 0; sp < n_splits; ++sp) mm = fmaxf(mm, get(sp).m);
+    float s = 0.0f, a = 0.0f, x = -__builtin_inff();
+    for (int sp = 0; sp < n_splits; ++sp) {  // fixed split order
+        const Partial p = get(sp);
+        const float f = fast_exp2((p.m - mm) * kLog2e);
+        const float ts = p.s * f, ta = p.pad * f;
+        s = s + ts;
+        a = a + ta;
+        x = fmaxf(x, p.xt);
+    }
+    const double lse = double(mm) + log2(double(s)) * kLn2;
+    if (entropy_slot != nullptr) *entropy_slot = float(lse - double(a) / double(s));  // -sum p log p = lse - sum p x
+    if (id < 0 || id >= vocab) {
+        *out_slot = __builtin_nanf("");
+        return;
+    }
+    *out_slot = float(double(x) - lse);
+}
+
+// One thread per row; the kernel before it has folded the units of every split.
 __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict__ partials,
                                                       const int64_t *__restrict__ ids, float *__restrict__ out,
                                                       float *__restrict__ entropy, int n_rows, int vocab, int n_splits) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= n_rows) return;
-    float mm = kFloor;
-    for (int sp = 0; sp < n_splits; ++sp) mm = fmaxf(mm, partials[size_t(sp) * n_rows + n].m);
-    float s = 0.0f, a = 0.0f, x = -__builtin_inff();
-    for (int sp = 0; sp < n_splits; ++sp) {  // fixed split order
-        const Partial p = partials[size_t(sp) * n_rows + n];
-        const float f = fast_exp2((p.m - mm) * kLog2e);
-        s += p.s * f;
-        a += p.pad * f;
-        x = fmaxf(x, p.xt);
+    lm_finish_row([&](int sp) { return partials[size_t(sp) * n_rows + n]; }, n_splits, ids[n], vocab, out + n,
+                  entropy != nullptr ? entropy + n : nullptr);
+}
+
+// Few rows: the kernel before it has written one partial per unit.  One wavefront per row: lane l folds the units of
+// the splits l, l + 64, ... in unit order (the same operations as the other kernel performs in place) into LDS, then
+// the splits are folded as above.
+constexpr int LM_FINE_MAX_SPLITS = 256;
+__global__ __launch_bounds__(256) void lmhead_combine_units(const Partial *__restrict__ partials,
+                                                            const int64_t *__restrict__ ids, float *__restrict__ out,
+                                                            float *__restrict__ entropy, int n_rows, int vocab,
+                                                            SplitPlan plan) {
+    __shared__ Partial folded[4][LM_FINE_MAX_SPLITS];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int n = blockIdx.x * 4 + wave;
+    if (n >= n_rows) return;  // wavefront-uniform; nothing below synchronises across wavefronts
+    const int n_splits = plan.n_splits;
+    for (int sp = lane; sp < n_splits; sp += kWave) {
+        float M = kFloor, S = 0.0f, X = -__builtin_inff(), A = 0.0f;
+        for (int j = 0; j < LM_SUBS; ++j) {
+            const int u = sp * LM_SUBS + j;
+            if (plan.unit_begin(u) == plan.unit_begin(u + 1)) continue;  // empty unit
+            const Partial p = partials[size_t(u) * n_rows + n];
+            lm_fold_unit(M, S, X, A, p.m, p.s, p.xt, p.pad);
+        }
+        Partial q;
+        q.m = M;
+        q.s = S;
+        q.xt = X;
+        q.pad = A;
+        folded[wave][sp] = q;
     }
-    const double lse = double(mm) + log2(double(s)) * kLn2;
-    if (entropy != nullptr) entropy[n] = float(lse - double(a) / double(s));  // -sum p log p = lse - sum p x
-    const int64_t id = ids[n];
-    if (id < 0 || id >= vocab) {
-        out[n] = __builtin_nanf("");
-        return;
-    }
-    out[n] = float(double(x) - lse);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (lane == 0)
+        lm_finish_row([&](int sp) { return folded[wave][sp]; }, n_splits, ids[n], vocab, out + n,
+                      entropy != nullptr ? entropy + n : nullptr);
 }
 
 inline int splits_for(int64_t vocab) {
     const int64_t n_vtiles = (vocab + LM_BM - 1) / LM_BM;
     return lm_n_splits(int(n_vtiles));
+}
+
+// Items are units instead of whole splits when whole splits would leave CUs without an item (the kernel runs one
+// workgroup on each of 256 CUs).  The choice changes the schedule and the size of the workspace, not a result bit.
+constexpr int LM_RESIDENT = 256;
+inline bool units_as_items(int64_t n_rows, int64_t vocab) {
+    const int64_t n_token_blocks = (n_rows + LM_BN - 1) / LM_BN;
+    const int n_splits = splits_for(vocab);
+    return n_token_blocks * n_splits < LM_RESIDENT && n_splits <= LM_FINE_MAX_SPLITS;
 }
 
 }  // namespace
@@ -571,7 +737,8 @@ inline int splits_for(int64_t vocab) {
 KA_EXPORT size_t ka_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab) {
     (void)hidden_dim;
     if (n_rows <= 0 || vocab <= 0) return 0;
-    return size_t(ka::splits_for(vocab)) * size_t(n_rows) * sizeof(ka::Partial);
+    const size_t per_row = size_t(ka::splits_for(vocab)) * (ka::units_as_items(n_rows, vocab) ? ka::LM_SUBS : 1);
+    return per_row * size_t(n_rows) * sizeof(ka::Partial);
 }
 
 namespace ka {
@@ -650,17 +817,19 @@ int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const
     const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
     const int n_splits = splits_for(vocab);
     const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
-    const int64_t n_virtual = ItemOrder(n_token_blocks, n_splits).n_virtual();
+    const int fine = units_as_items(n_rows, vocab) ? 1 : 0;
+    const SplitPlan plan(n_vtiles, n_splits);
+    const int64_t n_virtual = ItemOrder(n_token_blocks, plan, fine).n_virtual();
     if (n_virtual >= (int64_t(1) << 30)) return fail(KA_ERR_UNSUPPORTED, "lmhead: too many work items");
     // One workgroup per CU (a workgroup takes a CU's LDS and registers); each walks its items.  256 workgroups
     // keep item v on XCD v % 8 and at one position of its super-tiles.
-    const int64_t resident = dev.cus >= 256 ? 256 : (dev.cus >= 8 ? dev.cus / 8 * 8 : 8);
+    const int64_t resident = dev.cus >= LM_RESIDENT ? LM_RESIDENT : (dev.cus >= 8 ? dev.cus / 8 * 8 : 8);
     const int64_t grid = n_virtual < resident ? n_virtual : resident;
     const bool wide = n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32);
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                            static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
-                           int(n_rows), int(hidden_dim), int(vocab), n_splits, n_token_blocks, n_vtiles, int(n_virtual));
+                           int(n_rows), int(hidden_dim), int(vocab), n_token_blocks, plan, int(n_virtual), fine);
     };
     if (entropy != nullptr) {
         if (wide) launch(lmhead_partials<true, true>);
@@ -671,8 +840,12 @@ int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const
     }
     int rc = check_hip(hipGetLastError(), "lmhead partials launch");
     if (rc != KA_OK) return rc;
-    hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids, out,
-                       entropy, int(n_rows), int(vocab), n_splits);
+    if (fine)
+        hipLaunchKernelGGL(lmhead_combine_units, dim3(unsigned((n_rows + 3) / 4)), dim3(256), 0, stream, partials, ids,
+                           out, entropy, int(n_rows), int(vocab), plan);
+    else
+        hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids,
+                           out, entropy, int(n_rows), int(vocab), n_splits);
     return check_hip(hipGetLastError(), "lmhead combine launch");
 }
 

@@ -398,14 +398,7 @@ class SamplerBackend(nn.Module):
         lead = tuple(hidden.shape[:-1])
         if n_rows == 0:
             return (out.view(lead), ent.view(lead)) if return_entropy else out.view(lead)
-        # The workspace holds 16 B per row and vocabulary split; rows go to the kernel in slices that fit
-        # the pool (a multiple of the 256-token tile), which does not change any row's result.
-        per_row = self._lib.ka_lmhead_workspace_bytes(256, hdim, vocab) // 256
-        fit = self.pool.capacity // max(per_row, 1)
-        rows_per_call = n_rows if n_rows <= fit else fit // 256 * 256
-        if rows_per_call < 1:
-            raise PoolExhausted(f"the {self.pool.capacity} B pool cannot hold the lm_head partials of one "
-                                f"256-token tile ({256 * per_row} B)")
+        rows_per_call = self._lmhead_rows_per_call(n_rows, hdim, vocab)
         with _on_device(hidden.device):
             stream = _raw_stream()
             for start in range(0, n_rows, rows_per_call):
@@ -423,6 +416,22 @@ class SamplerBackend(nn.Module):
                             out.data_ptr() + start * 4, n, hdim, vocab, ws_ptr, ws_bytes, stream)
                 _hip.check(status, "ka_lmhead_logprob_bf16")
         return (out.view(lead), ent.view(lead)) if return_entropy else out.view(lead)
+
+    def _lmhead_rows_per_call(self, n_rows: int, hdim: int, vocab: int) -> int:
+        """Rows of one kernel call such that its partials fit the pool: all of them, or the largest multiple of the
+        256-token tile that fits (slicing the rows changes no row's result).  The workspace holds 16 B per row and
+        vocabulary split - four times that for calls of so few rows that the kernel spreads every split over four
+        workgroups - so the size is asked for, not computed here."""
+        need = self._lib.ka_lmhead_workspace_bytes
+        if need(n_rows, hdim, vocab) <= self.pool.capacity:
+            return n_rows
+        rows = self.pool.capacity // max(need(1 << 20, hdim, vocab) >> 20, 1) // 256 * 256
+        while rows >= 256 and need(rows, hdim, vocab) > self.pool.capacity:
+            rows -= 256
+        if rows < 256:
+            raise PoolExhausted(f"the {self.pool.capacity} B pool cannot hold the lm_head partials of one "
+                                f"256-token tile ({need(256, hdim, vocab)} B)")
+        return rows
 
     @torch.inference_mode()
     def fused_linear_logp_backward(self, hidden, weight, token_ids, grad_logp, chunk_tokens=None,

@@ -78,11 +78,14 @@ def test_lmhead_argument_checks_and_workspace_size():
     p = ctypes.c_void_p(4096)
     call = lib.ka_lmhead_logprob_bf16
     ws = lib.ka_lmhead_workspace_bytes
-    # 16 B per row and vocabulary split; the split count depends on the vocabulary only
+    # 16 B per row and vocabulary split; the split count depends on the vocabulary only.  Four times that (one
+    # partial per unit of a split) while token blocks x splits < 256: the call of few rows that spreads over all CUs
     assert ws(0, 4096, 128256) == 0
-    assert ws(1, 4096, 128256) == 16 * 64 and ws(32768, 4096, 128256) == 32768 * 16 * 64
-    assert ws(5, 64, 256) == 5 * 16 and ws(5, 64, 257) == 5 * 32 and ws(5, 64, 8 * 256) == 5 * 16 * 8
-    assert ws(5, 64, 9 * 256) == 5 * 16 * 8 and ws(5, 64, 65 * 256) == 5 * 16 * 16
+    assert ws(1, 4096, 128256) == 16 * 64 * 4 and ws(32768, 4096, 128256) == 32768 * 16 * 64
+    assert ws(768, 4096, 128256) == 768 * 16 * 64 * 4 and ws(769, 4096, 128256) == 769 * 16 * 64
+    assert ws(5, 64, 256) == 5 * 16 * 4 and ws(5, 64, 257) == 5 * 32 * 4 and ws(5, 64, 8 * 256) == 5 * 16 * 8 * 4
+    assert ws(5, 64, 9 * 256) == 5 * 16 * 8 * 4 and ws(5, 64, 65 * 256) == 5 * 16 * 16 * 4
+    assert ws(70000, 64, 9 * 256) == 70000 * 16 * 8
     assert ws(7, 64, 128256) == ws(7, 8192, 128256)
     assert call(None, None, None, None, 0, 4096, 128256, None, 0, None) == _hip.KA_OK             # no rows
     assert call(None, p, p, p, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG
@@ -91,12 +94,12 @@ def test_lmhead_argument_checks_and_workspace_size():
     assert call(ctypes.c_void_p(4100), p, p, p, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_UNSUPPORTED
     assert call(p, p, p, p, 4, 4096, 1 << 31, p, 1 << 40, None) == _hip.KA_ERR_UNSUPPORTED         # vocab of 2^31
     assert call(p, p, p, p, 4, 4096, 128256, None, 0, None) == _hip.KA_ERR_WORKSPACE
-    assert call(p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
+    assert call(p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 * 4 - 1, None) == _hip.KA_ERR_WORKSPACE
     assert b"workspace" in lib.ka_last_error()
     ent = lib.ka_lmhead_logprob_entropy_bf16
     assert ent(None, None, None, None, None, 0, 4096, 128256, None, 0, None) == _hip.KA_OK
     assert ent(p, p, p, p, None, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG           # entropy missing
-    assert ent(p, p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 - 1, None) == _hip.KA_ERR_WORKSPACE
+    assert ent(p, p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 * 4 - 1, None) == _hip.KA_ERR_WORKSPACE
     # the variant without a workspace argument: same checks, and a size limit instead of a workspace check
     na = lib.ka_lmhead_logprob_bf16_noalloc
     assert na(None, None, None, None, 0, 4096, 128256, None) == _hip.KA_OK

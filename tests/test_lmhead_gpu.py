@@ -89,8 +89,12 @@ def test_full_baseline_shape(sampler):
     pick = torch.randperm(32768, generator=torch.Generator().manual_seed(1))[:64].sort().values
     want = O.lmhead_logprob_ref(hidden[pick.cuda()].cpu(), weight.cpu(), ids[pick.cuda()].cpu(), dtype=torch.float32)
     assert (got[pick.cuda()].cpu() - want).abs().max().item() <= TOL
-    for lo, hi in ((0, 256), (20000, 20777)):
+    # calls of few rows run every split as four work items and fold them in the second kernel: same bits
+    for lo, hi in ((0, 64), (0, 256), (20000, 20600), (20000, 20777), (31000, 32768)):
         assert torch.equal(got[lo:hi], sampler.fused_linear_logp(hidden[lo:hi], weight, ids[lo:hi]))
+    lp, ent = sampler.fused_linear_logp(hidden[:8192], weight, ids[:8192], return_entropy=True)
+    lp64, ent64 = sampler.fused_linear_logp(hidden[100:164], weight, ids[100:164], return_entropy=True)
+    assert torch.equal(lp, got[:8192]) and torch.equal(lp64, got[100:164]) and torch.equal(ent64, ent[100:164])
 
 
 def test_weight_matrix_above_4_gib(sampler):
@@ -145,12 +149,13 @@ def test_rows_are_sliced_to_fit_a_small_workspace_pool(sampler):
     from rl_engine.kernels.sampling import SamplerBackend
 
     hidden, weight, ids = make(1000, 128, 40000, seed=9)
-    per_row = sampler._lib.ka_lmhead_workspace_bytes(256, 128, 40000) // 256   # 16 B per vocabulary split
+    per_row = sampler._lib.ka_lmhead_workspace_bytes(1 << 20, 128, 40000) >> 20   # 16 B per vocabulary split
     assert per_row % 16 == 0 and per_row >= 48
     base = sampler.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
-    small = SamplerBackend(pool_bytes=300 * per_row).cuda()              # room for 300 rows -> slices of 256
+    # (calls of so few rows keep one partial per unit of a split: four times per_row)
+    small = SamplerBackend(pool_bytes=4 * 300 * per_row).cuda()          # room for 300 rows -> slices of 256
     assert torch.equal(small.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda()), base)
-    tiny = SamplerBackend(pool_bytes=100 * per_row).cuda()                    # less than one tile of a long input
+    tiny = SamplerBackend(pool_bytes=4 * 100 * per_row).cuda()                # less than one tile of a long input
     with pytest.raises(PoolExhausted):
         tiny.fused_linear_logp(hidden.cuda(), weight.cuda(), ids.cuda())
     assert torch.equal(tiny.fused_linear_logp(hidden[:64].cuda(), weight.cuda(), ids[:64].cuda()), base[:64])

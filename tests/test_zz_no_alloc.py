@@ -77,7 +77,7 @@ def test_noalloc_entry_rejects_what_does_not_fit():
     dev = torch.device("cuda", 0)
     limit = _hip.LMHEAD_STATIC_SCRATCH_BYTES
     h, v = 64, 128256
-    fits = limit // (lib.ka_lmhead_workspace_bytes(1, h, v))
+    fits = limit // (lib.ka_lmhead_workspace_bytes(1 << 20, h, v) >> 20)   # bytes per row of a call of many rows
     assert lib.ka_lmhead_workspace_bytes(fits, h, v) <= limit < lib.ka_lmhead_workspace_bytes(fits + 1, h, v)
     assert fits == 16384
     # real (small) buffers, a row count beyond the limit: the call must refuse before it launches anything
