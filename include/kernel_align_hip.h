@@ -37,8 +37,17 @@ extern "C" {
 #define KA_DTYPE_F16 1
 #define KA_DTYPE_F32 2
 
-/* Library version string, e.g. "kernel_align_hip 0.1 (gfx950)". */
+/* Library version string, e.g. "kernel_align_hip 0.3 (gfx950)". */
 const char *ka_version(void);
+/*
+ * Revision of this interface: raised whenever the signature or the meaning of an entry point changes.  A binding
+ * compares ka_abi_revision() with the KA_ABI_REVISION it was written against and refuses a library that differs (a
+ * caller bound to another prototype would pass its arguments in the wrong places without any error).
+ * Result bits of the floating-point operators (fixed summation orders) are stable within one revision of the library,
+ * not across revisions; token ids are defined exactly and never change.
+ */
+#define KA_ABI_REVISION 3
+int ka_abi_revision(void);
 /* Message of the last error on the calling thread ("" if none). */
 const char *ka_last_error(void);
 /* Name of a status code. */
@@ -161,7 +170,8 @@ int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, in
  * flags (0 in production) selects among routes that compute the same function, so that a caller can check one
  * against the other: KA_SAMPLE_FLAG_GENERAL_PATH runs the general radix-select path even where a shorter route
  * applies; KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK keeps the top-k route on its block-wide selection and tail instead of the
- * wavefront-local ones it takes for top_k <= 64.  Ids and log-probabilities do not depend on the flags.
+ * short ones it takes for top_k <= 256 (bound from pooled maxima up to top_k = 64, from a radix descent above).  Ids
+ * and log-probabilities do not depend on the flags.
  */
 #define KA_SAMPLE_FLAG_GENERAL_PATH 1u
 #define KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK 2u
@@ -187,8 +197,10 @@ int ka_sample_mass_fixed(const float *d, int64_t n, uint64_t *out, void *hip_str
  * row-major (the nn.Linear.weight layout).  bf16 MFMA with fp32 accumulation;
  * logit tiles stay in registers and feed an online max / log-sum-exp.
  * hidden_dim must be a multiple of 64 and both matrices 16-byte aligned; the
- * workspace (16 bytes per row and vocabulary split, as the query reports) must
- * be 16-byte aligned.  A row's result does not depend on n_rows.  An id outside
+ * workspace (as the query reports: 16 bytes per row and vocabulary split, four
+ * times that for calls of so few rows - token blocks x splits < 256 - that every
+ * split is spread over four workgroups to fill the part) must be 16-byte
+ * aligned.  A row's result does not depend on n_rows, bit for bit.  An id outside
  * [0, vocab) gives NaN for its row.  The kernel is launched as one workgroup
  * per CU, each walking its share of the work.
  * No counterpart in the reference; the nearest behaviour is
@@ -215,7 +227,7 @@ int ka_lmhead_logprob_entropy_bf16(const void *hidden, const void *weight, const
  * one copy on every GPU the library runs on, held until the process ends) instead of a workspace, and the
  * call makes no hipMalloc / hipFree.  It has no counterpart in the reference.
  * Limit: ka_lmhead_workspace_bytes(n_rows, hidden_dim, vocab) <= KA_LMHEAD_STATIC_SCRATCH_BYTES (16,384
- * rows at a vocabulary of 128,256); more returns KA_ERR_WORKSPACE and nothing is launched.  Every call on
+ * rows at a vocabulary of 128,256: 16 MiB; up to 768 rows the same vocabulary takes 64 KiB per row: 3 MiB); more returns KA_ERR_WORKSPACE and nothing is launched.  Every call on
  * a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on
  * one stream are ordered and safe.  The first call on a device looks the array's address up (one
  * hipGetSymbolAddress and the kernels' attribute set-up), so make one call per device before capturing.

@@ -164,10 +164,7 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
     // compile-time 1, which keeps their kernels as they are).  (A resident row keeps no per-vector maxima: with the
     // row in 64 registers of the 128 a lane has, sixteen more spill and slow the read down.)
     constexpr int TRK_VECS = 32;
-#ifndef KA_TRK_BATCH
-#define KA_TRK_BATCH 8
-#endif
-    constexpr int TRK_BATCH = KA_TRK_BATCH;  // loads in flight per lane (with 16, the 128 registers of a lane spill)
+    constexpr int TRK_BATCH = 8;  // loads in flight per lane (with 16, the 128 registers of a lane spill)
     const int trk_need = (nvec + TRK_VECS * S_THREADS - 1) / (TRK_VECS * S_THREADS);
     const int trk_rounds = T::kBytes == 4 ? trk_need : 1;
     const bool tracked = vec && !resident && trk_need <= (T::kBytes == 4 ? 4 : 1);

@@ -16,6 +16,9 @@ KA_ERR_UNSUPPORTED = -2
 KA_ERR_WORKSPACE = -3
 KA_ERR_HIP = -4
 
+# Revision of include/kernel_align_hip.h that the signatures below were written against (KA_ABI_REVISION).
+ABI_REVISION = 3
+
 LIB_NAME = "libkernel_align_hip.so"
 ENV_LIB = "KERNEL_ALIGN_HIP_LIB"
 
@@ -28,6 +31,7 @@ _SAMPLE_ARGS = [c_void_p, c_int64, c_int64, c_int64, c_float, c_int32, c_float, 
 # name -> (restype, argtypes); must list every symbol the header declares.
 SIGNATURES = {
     "ka_version": (c_char_p, []),
+    "ka_abi_revision": (c_int, []),
     "ka_last_error": (c_char_p, []),
     "ka_status_string": (c_char_p, [c_int]),
     "ka_logprob_bf16": (c_int, _LOGPROB_ARGS),
@@ -101,6 +105,10 @@ def load() -> ctypes.CDLL:
             raise HipLibraryError(f"{path} does not export {name}") from exc
         fn.restype = restype
         fn.argtypes = argtypes
+    found = lib.ka_abi_revision()
+    if found != ABI_REVISION:
+        raise HipLibraryError(f"{path} implements interface revision {found}, this binding was written against "
+                              f"revision {ABI_REVISION}: rebuild the library (python kernel-align_amd/build_hip.py)")
     _lib = lib
     return lib
 

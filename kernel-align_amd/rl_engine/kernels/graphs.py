@@ -14,6 +14,12 @@ that the operators can be captured at all.
     step.uniforms.copy_(torch.rand(64))
     ids, logp = step()                      # tensors owned by the step, overwritten by the next replay
 
+Which operators may be captured: all of them.  compute_logp, compute_logp_entropy, compute_logp_backward, grpo_token_loss
+and sample need no scratch memory.  fused_linear_logp does: under capture its partial results go to memory allocated by
+the capture itself (the graph's own pool), not to the backend's shared arena, so a replay can run while eager calls on
+other streams use the arena (rl_engine/kernels/pool.py).  Tensors that an operator returns under capture are owned by
+the graph and overwritten by every replay.
+
 The reference has no counterpart (its operators are plain eager calls, rl_engine/kernels/sampling.py:39-112).
 """
 from __future__ import annotations

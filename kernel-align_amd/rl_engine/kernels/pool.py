@@ -15,6 +15,14 @@ hold the same bytes, and every lease leaves an event on the stream it was used
 on.  A later lease on another stream first makes that stream wait for the event,
 so kernels of two streams never work in the arena at the same time (they run one
 after the other; results are those of sequential calls).
+
+HIP-graph capture.  A lease taken while the current stream is capturing does not
+touch the arena or the events (waiting for an event recorded outside the capture,
+or leaving a capture-recorded event for eager streams, is not valid, and a replay
+would use the arena without any ordering against eager calls): it hands out memory
+allocated under the capture, which belongs to the graph's own memory pool.  A
+captured operator therefore owns its scratch; replays of the graph and eager calls
+on other streams never share bytes.
 """
 from __future__ import annotations
 
@@ -78,6 +86,12 @@ class WorkspacePool:
         docstring): the whole arena is taken, the previous user's stream is waited for, and the lock is
         released only after this user's event is recorded."""
         index = device.index if device.index is not None else torch.cuda.current_device()
+        if torch.cuda.is_current_stream_capturing():
+            if nbytes > self.capacity:
+                raise PoolExhausted(f"workspace request of {nbytes} B exceeds the {self.capacity} B pool size")
+            # graph-private memory: lives as long as the graph, used by its replays only
+            yield torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=torch.device("cuda", index))[:nbytes]
+            return
         with self._lock:
             self.reset()
             view = self.reserve(nbytes, device)

@@ -26,6 +26,20 @@ def test_header_binding_and_library_agree():
         assert getattr(lib, name) is not None
 
 
+def test_interface_revision_is_checked(monkeypatch):
+    """The header, the binding and the library carry the same interface revision, and a binding written against
+    another revision refuses the library instead of calling it with arguments in the wrong places."""
+    lib = _hip.load()
+    header_rev = int(re.search(r"#define KA_ABI_REVISION (\d+)", HEADER.read_text()).group(1))
+    assert lib.ka_abi_revision() == header_rev == _hip.ABI_REVISION
+    monkeypatch.setattr(_hip, "_lib", None)
+    monkeypatch.setattr(_hip, "ABI_REVISION", header_rev + 1)
+    with pytest.raises(_hip.HipLibraryError, match="interface revision"):
+        _hip.load()
+    monkeypatch.setattr(_hip, "ABI_REVISION", header_rev)
+    assert _hip.load().ka_abi_revision() == header_rev
+
+
 def test_version_and_status_strings():
     lib = _hip.load()
     assert b"gfx950" in lib.ka_version()

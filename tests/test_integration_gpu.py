@@ -167,3 +167,98 @@ def test_policy_logprob_from_the_sampling_call(sampler):
         assert torch.equal(torch.cat(parts), policy1)
     e_ids, e_pol = sampler.sample(torch.empty(0, 100, dtype=torch.bfloat16, device="cuda"), return_policy_logprob=True)
     assert e_ids.numel() == 0 and e_pol.numel() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_policy_logprob_on_rows_that_start_with_masked_entries(sampler, dtype):
+    """The log-sum-exp that the sampling kernel takes along uses the same floor-started running maximum as the logprob
+    kernel: a masked prefix (a lane's first entries are all -inf), every other entry masked, a single finite entry at
+    the end of the row.  At the headline row length, on every route, against compute_logp (1e-5) and the oracle (1e-4)."""
+    from oracle import logprob_ref
+    from rl_engine.kernels import _hip
+
+    g = torch.Generator().manual_seed(83)
+    host = (torch.randn(10, 128256, generator=g) * 3).to(dtype)
+    host[0, :70000] = float("-inf")
+    host[1, :1000] = float("-inf")
+    host[2, 1::2] = float("-inf")
+    host[3, :] = float("-inf")
+    host[3, 128255] = 1.0
+    host[4, :128000] = float("-inf")                                     # fewer finite entries than top_k = 500
+    logits, u = host.cuda(), torch.rand(10, generator=g).cuda()
+    for kw in (dict(top_k=50, top_p=0.9, temperature=0.7), dict(top_k=200), dict(top_k=500, top_p=0.95), dict(top_p=0.9),
+               dict()):
+        for flags in (0, _hip.SAMPLE_FLAG_BLOCK_WIDE_TOPK, _hip.SAMPLE_FLAG_GENERAL_PATH):
+            ids, policy = sampler.sample(logits, uniforms=u, return_policy_logprob=True, route_flags=flags, **kw)
+            assert torch.equal(ids.cpu(), exact.sample(host, kw.get("temperature", 1.0), kw.get("top_k"), kw.get("top_p"), u.cpu()))
+            assert torch.isfinite(policy).all(), (dtype, kw, flags)
+            assert (policy - sampler.compute_logp(logits, ids)).abs().max().item() <= 1e-5, (dtype, kw, flags)
+            assert (policy.cpu() - logprob_ref.logprob_ref(host, ids.cpu())).abs().max().item() <= 1e-4
+            assert ids[3].item() == 128255 and abs(policy[3].item()) <= 1e-6
+
+
+def test_policy_logprob_at_the_benchmark_shape_and_with_per_row_parameters(sampler):
+    """bf16 [256, 128256] as the sampling benchmark draws it: ids against the oracle, the policy log-probability against
+    compute_logp and the oracle; then one call with per-row top_k / top_p / temperature tensors (the kernel variant
+    with the dense-histogram LDS, whose routes pass over the row once more for the log-sum-exp) and a ragged fp32 row
+    length that takes several tracking rounds."""
+    from benchmarks.workloads import cfg5_sampling
+    from oracle import logprob_ref
+
+    host, u = cfg5_sampling(256)
+    logits, ug = host.cuda(), u.cuda()
+    ids, policy = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=ug, return_policy_logprob=True)
+    assert torch.equal(ids.cpu(), exact.sample(host, 0.7, 50, 0.9, u))
+    assert (policy - sampler.compute_logp(logits, ids)).abs().max().item() <= 1e-5
+    assert (policy.cpu() - logprob_ref.logprob_ref(host, ids.cpu())).abs().max().item() <= 1e-4
+    g = torch.Generator().manual_seed(84)
+    k_rows = torch.randint(0, 3000, (256,), generator=g).to(torch.int32)          # 0 = off; beyond 1024: dense histogram
+    k_rows[:32] = torch.randint(1, 64, (32,), generator=g).to(torch.int32)
+    p_rows = torch.rand(256, generator=g) * 0.6 + 0.4
+    p_rows[::7] = 1.0
+    t_rows = torch.rand(256, generator=g) * 1.5 + 0.25
+    ids2, policy2 = sampler.sample(logits, top_k=k_rows.cuda(), top_p=p_rows.cuda(), temperature=t_rows.cuda(),
+                                   uniforms=ug, return_policy_logprob=True)
+    want = exact.sample_rows(host, t_rows, k_rows, p_rows, u)[0]
+    assert torch.equal(ids2.cpu(), want)
+    assert (policy2 - sampler.compute_logp(logits, ids2)).abs().max().item() <= 1e-5
+    assert (policy2.cpu() - logprob_ref.logprob_ref(host, ids2.cpu())).abs().max().item() <= 1e-4
+    wide = (torch.randn(6, 300003, generator=g) * 3)                              # fp32, ragged, three tracking rounds
+    wide[1, :150000] = float("-inf")
+    uw = torch.rand(6, generator=g)
+    ids3, policy3 = sampler.sample(wide.cuda(), top_k=40, top_p=0.9, temperature=0.8, uniforms=uw.cuda(),
+                                   return_policy_logprob=True)
+    assert torch.equal(ids3.cpu(), exact.sample(wide, 0.8, 40, 0.9, uw))
+    assert (policy3.cpu() - logprob_ref.logprob_ref(wide, ids3.cpu())).abs().max().item() <= 1e-4
+
+
+def test_captured_fused_linear_logp_owns_its_workspace(sampler):
+    """A fused_linear_logp captured in a HIP graph takes its scratch from the graph's own memory, not from the backend's
+    arena: replays on one stream run while eager calls (which lease the arena) run on another, and both results stay
+    bit-equal to sequential calls.  The two inputs are sized so that their partial results would overlap in the arena."""
+    def make(n, seed):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        return (torch.randn(n, 512, generator=g, device="cuda").bfloat16(),
+                (torch.randn(30000, 512, generator=g, device="cuda") * 0.05).bfloat16(),
+                torch.randint(0, 30000, (n,), generator=g, device="cuda"))
+
+    a, b = make(2048, 41), make(1792, 42)
+    want_a, want_b = sampler.fused_linear_logp(*a), sampler.fused_linear_logp(*b)
+    torch.cuda.synchronize()
+    arena_before = sampler.pool._last_use.get(0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got_a = sampler.fused_linear_logp(*a)
+    assert sampler.pool._last_use.get(0) is arena_before          # the capture left no event behind in the pool
+    side = torch.cuda.Stream()
+    for _ in range(4):
+        with torch.inference_mode():
+            got_a.zero_()
+        torch.cuda.synchronize()
+        graph.replay()                                             # on the current stream
+        with torch.cuda.stream(side):
+            got_b = [sampler.fused_linear_logp(*b) for _ in range(3)]  # eager, arena, other stream, concurrently
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got_a, want_a)
+        assert all(torch.equal(x, want_b) for x in got_b)

@@ -97,6 +97,25 @@ def test_entropy_closed_forms():
     assert O.entropy_f64(x).item() == 0.0
 
 
+def test_entropy_against_a_pure_python_evaluation():
+    """Rows that are neither uniform nor one-hot, evaluated term by term with math.fsum: a weighting that only the two
+    closed forms above cannot tell from the right one (p * x without the log-sum-exp, a missing sign, log2 for log)
+    fails here."""
+    rows = [[0.5, -1.25, 3.0, 0.0, 2.0, -0.75, 1.5],
+            [-3.0, -3.0, 4.0, 4.0, -math.inf, 0.25, 10.0, -8.0],
+            [20.0, 19.5, -20.0]]
+    for row in rows:
+        m = max(row)
+        z = math.fsum(math.exp(x - m) for x in row)
+        probs = [math.exp(x - m) / z for x in row]
+        want = -math.fsum(p * math.log(p) for p in probs if p > 0.0)
+        got = O.entropy_f64(torch.tensor([row], dtype=torch.float32)).item()
+        assert abs(got - want) < 1e-12, (row, got, want)
+        assert 0.0 < want < math.log(len(row))
+    # two equal entries and nothing else: exactly ln 2, whatever their common value
+    assert abs(O.entropy_f64(torch.tensor([[-math.inf, 7.0, 7.0, -math.inf]])).item() - math.log(2.0)) < 1e-15
+
+
 def test_backward_closed_form_is_autograd():
     g = torch.Generator().manual_seed(0)
     logits = torch.randn(16, 999, generator=g) * 3
