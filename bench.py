@@ -31,19 +31,43 @@ BYTES_PER_TOKEN = 2 * V + 8 + 4
 # what the counters read for a plain 1 GiB copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000), and
 # are repeated here with their source so that a reader can tell them from live figures.  A kernel whose code
 # changed after its profile was taken reports null until the profile is redone.
+# Each entry: bytes per launch, the profile that records the counter runs, the kernel's source files, and the first 16
+# hex digits of the SHA-256 of those files (concatenated in that order) at the time of the counter runs.
+CSRC = REPO / "kernel-align_amd" / "csrc"
+_SAMPLING_SOURCES = ("ka_common.h", "ka_sampling_common.h", "ka_sampling_topk.h", "ka_sampling_dense.h", "ka_sampling_draw.h",
+                     "ka_sampling.hip")
 STATIC_TRAFFIC = {
-    "logprob_rows": ((2 * 1026607.7 + 258.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt"),
-    "logprob_backward_rows": ((2 * 1027116 + 2052133) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt"),
-    "sample_rows": ((2 * 32796.6 + 8) * 1024, "profiles/sample_rows_bf16_B64-256_V128256.txt"),                       # B = 256
-    "lmhead_partials": ((2 * 3.19204e7 + 79071.5) * 1024, "profiles/lmhead_partials_bf16_N32768_H4096_V128256.txt"),  # L2 misses: varies +-30 % between calls
+    "logprob_rows": ((2 * 1026607.7 + 258.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",
+                     ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
+    "logprob_backward_rows": ((2 * 1027116 + 2052133) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",
+                              ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
+    "sample_rows": ((2 * 32796.6 + 8) * 1024, "profiles/sample_rows_bf16_B64-1024_V128256.txt",                      # B = 256
+                    _SAMPLING_SOURCES, "@SHA_SAMPLING@"),
+    "lmhead_partials": ((2 * 3.19204e7 + 79071.5) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt",         # N = 32768; L2 misses: varies +-30 % between calls
+                        ("ka_common.h", "ka_lmhead.hip"), "@SHA_LMHEAD@"),
 }
 PARITY_TOL = 1e-4
 
 
-def traffic_fields(kernel: str) -> dict:
-    value, source = STATIC_TRAFFIC[kernel]
-    return {"traffic": value, "traffic_source": f"static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in {source}"
-            if value is not None else "not collected for the current build of this kernel"}
+def source_fingerprint(files) -> str:
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in files:
+        h.update((CSRC / name).read_bytes())
+    return h.hexdigest()[:16]
+
+
+def traffic_fields(kernel: str, scale: float = 1.0) -> dict:
+    """The recorded counter traffic of `kernel` (times `scale`), or null when the kernel's sources are no longer the
+    ones the counter runs were taken from."""
+    value, source, files, sha = STATIC_TRAFFIC[kernel]
+    now = source_fingerprint(files)
+    if now != sha:
+        return {"traffic": None, "traffic_source": f"not collected for this build of the kernel (sources {now}, counter runs "
+                                                   f"in {source} were taken from {sha})"}
+    return {"traffic": value * scale,
+            "traffic_source": f"static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded in {source} (sources {sha})"}
 
 
 def log(msg: str) -> None:
@@ -95,8 +119,9 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
     import torch
     from benchmarks.workloads import cfg5_sampling
 
-    out = {"config": "bf16 [B,128256] ~ N(0,3^2), T=0.7, top_k=50, top_p=0.9, one fp32 uniform per row (seed 1234)"}
-    for batch in (64, 128, 256):
+    out = {"config": "bf16 [B,128256] ~ N(0,3^2), T=0.7, top_k=50, top_p=0.9, one fp32 uniform per row (seed 1234)",
+           "roofline_by_batch": {}}
+    for batch in (64, 128, 256, 512, 1024):
         logits, u = cfg5_sampling(batch, device="cuda")
         for _ in range(max(warmup, 3)):
             sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u)
@@ -127,7 +152,16 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
         torch.cuda.synchronize()
         kernel_ms = ev0.elapsed_time(ev1) / 200
         out[f"kernel_ms_b{batch}"] = kernel_ms
-        # a decode step: the id and its log-probability under the unfiltered softmax from the one kernel
+        gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
+        out["roofline_by_batch"][f"b{batch}"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                                 "frac": gbps / HBM_PEAK_GBPS, "kernel_ms": kernel_ms,
+                                                 "bytes_per_launch": batch * BYTES_PER_TOKEN}
+        # a decode step: the id and its log-probability under the unfiltered softmax from the one kernel; checked once
+        # against the logprob operator on the drawn ids before it is timed
+        d_ids, d_pol = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+        d_err = (d_pol - sampler.compute_logp(logits, d_ids)).abs().max().item()
+        out[f"decode_step_policy_max_abs_diff_b{batch}"] = d_err
+        assert d_err <= 1e-5, f"decode step: policy log-probability differs from compute_logp by {d_err}"
         for _ in range(5):
             sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
         torch.cuda.synchronize()
@@ -138,7 +172,6 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
         torch.cuda.synchronize()
         out[f"decode_step_ms_b{batch}"] = ev0.elapsed_time(ev1) / 100
         if batch == 256:
-            gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                "frac": gbps / HBM_PEAK_GBPS, **traffic_fields("sample_rows"), "kernel": "sample_rows<Bf16>"}
             # the other filter combinations at the same batch (kernel time per call, microseconds)
@@ -229,10 +262,32 @@ def lmhead_throughput(sampler, iters: int = 3):
     ms = ev0.elapsed_time(ev1) / iters
     tflops = 2.0 * n * h * v / (ms * 1e-3) / 1e12
     assert bool(torch.isfinite(out).all())
+    # Decode-sized calls (the call in front of a sampling step): one token block, bound by streaming W once from HBM.
+    decode = {}
+    w_bytes = v * h * 2
+    for rows in (64, 256):
+        hs, is_ = hidden[:rows], ids[:rows]
+        assert torch.equal(sampler.fused_linear_logp(hs, weight, is_), out[:rows]), "a row's result depends on the row count"
+        for _ in range(3):
+            sampler.fused_linear_logp(hs, weight, is_)
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(20):
+            sampler.fused_linear_logp(hs, weight, is_)
+        ev1.record()
+        torch.cuda.synchronize()
+        ms_small = ev0.elapsed_time(ev1) / 20
+        alg = w_bytes + rows * (h * 2 + 8 + 4)
+        gbps = alg / (ms_small * 1e-3) / 1e9
+        decode[f"n{rows}"] = {"ms": ms_small, "bit_identical_to_the_rows_of_the_large_call": True,
+                              "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                           "frac": gbps / HBM_PEAK_GBPS, "bytes_per_call": alg, "traffic": None,
+                                           "kernel": "lmhead_partials (units as work items) + lmhead_combine_units"}}
     return {"config": "hidden bf16 [32768,4096] ~ N(0,1), W bf16 [128256,4096] ~ N(0,0.02^2), seed 0; logits never stored",
             "ms": ms, "tokens_per_s": n / (ms * 1e-3),
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s",
-                         "frac": tflops / 2500.0, **traffic_fields("lmhead_partials"), "kernel": "lmhead_partials"}}
+                         "frac": tflops / 2500.0, **traffic_fields("lmhead_partials"), "kernel": "lmhead_partials"},
+            "decode_sized": decode}
 
 
 def main() -> int:
@@ -259,6 +314,7 @@ def main() -> int:
     for handler in logger.handlers:  # stdout carries the JSON line only
         handler.setStream(sys.stderr)
     from benchmarks.workloads import spike_logits
+    from rl_engine.kernels import _hip as _hip_mod
     from rl_engine.kernels import sampling as sampling_mod
     from rl_engine.kernels.sampling import SamplerBackend
 
@@ -331,10 +387,13 @@ def main() -> int:
         "hbm_gbps": n_rows * BYTES_PER_TOKEN / (ms_per_step * 1e-3) / 1e9,
         "extra_device_bytes": extra_device_bytes,
         "resident_bytes": resident,
+        # what the library holds on the device whatever is called: the static array behind
+        # ka_lmhead_logprob_bf16_noalloc (loaded with the code object) and, once fused_linear_logp has run, the pool arena
+        "library_static_scratch_bytes": _hip_mod.LMHEAD_STATIC_SCRATCH_BYTES,
+        "pool_capacity_bytes": sampler.pool.capacity,
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS,
-                     "traffic": STATIC_TRAFFIC["logprob_rows"][0] * rows_per_launch / 8192,
-                     "traffic_source": traffic_fields("logprob_rows")["traffic_source"],
+                     **traffic_fields("logprob_rows", rows_per_launch / 8192),
                      "kernel": "logprob_rows<Bf16,256,4,vec>", "launch_ms": launch_ms,
                      "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
     }
@@ -348,6 +407,7 @@ def main() -> int:
     result["sampling"] = sampling_latency(sampler, args.steps, args.warmup, cpu=args.cpu_sample_rows > 0)
     if not args.skip_lmhead:
         result["fused_lm_head"] = lmhead_throughput(sampler)
+    result["pool_allocated_bytes_at_exit"] = sampler.pool.allocated_bytes()
     print(json.dumps(result), flush=True)
     parity = result.get("cpu_baseline", {}).get("parity")
     if parity is not None and not parity["ok"]:
