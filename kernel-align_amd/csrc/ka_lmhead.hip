@@ -646,6 +646,14 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the trailing (redundant) slab copies still write LDS
 }
 
+}  // namespace
+}  // namespace ka
+
+#include "ka_lmhead_narrow.h"
+
+namespace ka {
+namespace {
+
 // The fold of a row's split partials, in split order, and the two results.  get(sp) returns the partial of split sp.
 // Written out operation by operation (no contraction): whoever produced the split partials, the bits are the same.
 template <typename Get>
@@ -725,6 +733,10 @@ inline int splits_for(int64_t vocab) {
 // Items are units instead of whole splits when whole splits would leave CUs without an item (the kernel runs one
 // workgroup on each of 256 CUs).  The choice changes the schedule and the size of the workspace, not a result bit.
 constexpr int LM_RESIDENT = 256;
+// Up to this many rows a call runs the kernel of ka_lmhead_narrow.h (64 tokens per workgroup up to 64 rows, 128 above).
+// (Measured at V = 128,256, H = 4096: 64 rows 0.27 -> 0.20 ms, 128 rows 0.27 -> 0.21 ms; 256 rows as two 128-token blocks
+// 0.35 ms against 0.30 ms for the 256-token kernel, so the limit stays at one 128-token block.)
+constexpr int LN_MAX_ROWS = 128;
 inline bool units_as_items(int64_t n_rows, int64_t vocab) {
     const int64_t n_token_blocks = (n_rows + LM_BN - 1) / LM_BN;
     const int n_splits = splits_for(vocab);
@@ -780,7 +792,19 @@ int lm_current_device(bool need_scratch, LmDevice &out) {
                                   reinterpret_cast<const void *>(lmhead_partials<true, true>)};
         for (int k = 0; k < 4 && rc == hipSuccess; ++k)
             rc = hipFuncSetAttribute(kernels[k], hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
-        if (rc != hipSuccess) return check_hip(rc, "lmhead: reserving 131 KB of LDS");
+        if (rc == hipSuccess)
+            rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials_narrow<1, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, ln_lds_bytes<1>());
+        if (rc == hipSuccess)
+            rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials_narrow<1, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, ln_lds_bytes<1>());
+        if (rc == hipSuccess)
+            rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials_narrow<2, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, ln_lds_bytes<2>());
+        if (rc == hipSuccess)
+            rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials_narrow<2, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, ln_lds_bytes<2>());
+        if (rc != hipSuccess) return check_hip(rc, "lmhead: reserving LDS for the kernels");
         d.cus = cus;
         d.ready = true;
     }
@@ -826,6 +850,30 @@ int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const
     const int64_t resident = dev.cus >= LM_RESIDENT ? LM_RESIDENT : (dev.cus >= 8 ? dev.cus / 8 * 8 : 8);
     const int64_t grid = n_virtual < resident ? n_virtual : resident;
     const bool wide = n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32);
+    if (fine && !wide && n_rows <= LN_MAX_ROWS) {
+        // Few rows: the kernel with 64- or 128-token workgroups and three stages of slabs (ka_lmhead_narrow.h).
+        const int tn = n_rows <= 64 ? 1 : 2;
+        const int ntb = int((n_rows + 64 * tn - 1) / (64 * tn));
+        const int64_t nvirt = ItemOrder(ntb, plan, 1).n_virtual();
+        const int64_t g = nvirt < resident ? nvirt : resident;
+        auto go = [&](auto kernel, int lds_bytes) {
+            hipLaunchKernelGGL(kernel, dim3(unsigned(g)), dim3(LM_THREADS), lds_bytes, stream,
+                               static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
+                               int(n_rows), int(hidden_dim), int(vocab), ntb, plan, int(nvirt));
+        };
+        if (tn == 1) {
+            if (entropy != nullptr) go(lmhead_partials_narrow<1, true>, ln_lds_bytes<1>());
+            else go(lmhead_partials_narrow<1, false>, ln_lds_bytes<1>());
+        } else {
+            if (entropy != nullptr) go(lmhead_partials_narrow<2, true>, ln_lds_bytes<2>());
+            else go(lmhead_partials_narrow<2, false>, ln_lds_bytes<2>());
+        }
+        const int rcn = check_hip(hipGetLastError(), "lmhead partials launch (few rows)");
+        if (rcn != KA_OK) return rcn;
+        hipLaunchKernelGGL(lmhead_combine_units, dim3(unsigned((n_rows + 3) / 4)), dim3(256), 0, stream, partials, ids,
+                           out, entropy, int(n_rows), int(vocab), plan);
+        return check_hip(hipGetLastError(), "lmhead combine launch");
+    }
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                            static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
