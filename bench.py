@@ -36,16 +36,21 @@ BYTES_PER_TOKEN = 2 * V + 8 + 4
 CSRC = REPO / "kernel-align_amd" / "csrc"
 _SAMPLING_SOURCES = ("ka_common.h", "ka_sampling_common.h", "ka_sampling_topk.h", "ka_sampling_dense.h", "ka_sampling_draw.h",
                      "ka_sampling.hip")
+_LMHEAD_SOURCES = ("ka_common.h", "ka_lmhead.hip", "ka_lmhead_narrow.h")
 STATIC_TRAFFIC = {
     "logprob_rows": ((2 * 1026607.7 + 258.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",
                      ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
     "logprob_backward_rows": ((2 * 1027116 + 2052133) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",
                               ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
-    "sample_rows": ((2 * 32796.6 + 8) * 1024, "profiles/sample_rows_bf16_B64-1024_V128256.txt",                      # B = 256
-                    _SAMPLING_SOURCES, "@SHA_SAMPLING@"),
-    "lmhead_partials": ((2 * 3.19204e7 + 79071.5) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt",         # N = 32768; L2 misses: varies +-30 % between calls
-                        ("ka_common.h", "ka_lmhead.hip"), "@SHA_LMHEAD@"),
+    "sample_rows": ((2 * 32846.4 + 10.3) * 1024, "profiles/sample_rows_bf16_B64-1024_V128256.txt",                     # B = 256
+                    _SAMPLING_SOURCES, "3b612db1d4536cb9"),
+    "lmhead_partials": ((2 * 2.998e7 + 121088) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt",            # N = 32768; L2 misses: varies +-50 % between calls
+                        _LMHEAD_SOURCES, "aa1c04c3ec8bc5a7"),
+    "lmhead_n64": ((2 * 517356 + 256) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt", _LMHEAD_SOURCES, "aa1c04c3ec8bc5a7"),
+    "lmhead_n256": ((2 * 532238 + 9216) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt", _LMHEAD_SOURCES, "aa1c04c3ec8bc5a7"),
 }
+# FETCH_SIZE / WRITE_SIZE KiB per dispatch of sample_rows by batch, from the same counter runs as the B = 256 entry above
+_SAMPLING_KIB = {64: (8282.9, 2.6), 128: (16329.9, 5.3), 256: (32846.4, 10.3), 512: (65465.0, 21.0), 1024: (130680.0, 42.1)}
 PARITY_TOL = 1e-4
 
 
@@ -155,7 +160,9 @@ def sampling_latency(sampler, steps: int, warmup: int, cpu: bool = True):
         gbps = batch * BYTES_PER_TOKEN / (kernel_ms * 1e-3) / 1e9
         out["roofline_by_batch"][f"b{batch}"] = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                                  "frac": gbps / HBM_PEAK_GBPS, "kernel_ms": kernel_ms,
-                                                 "bytes_per_launch": batch * BYTES_PER_TOKEN}
+                                                 "bytes_per_launch": batch * BYTES_PER_TOKEN,
+                                                 **traffic_fields("sample_rows", (2 * _SAMPLING_KIB[batch][0] + _SAMPLING_KIB[batch][1])
+                                                                  / (2 * _SAMPLING_KIB[256][0] + _SAMPLING_KIB[256][1]))}
         # a decode step: the id and its log-probability under the unfiltered softmax from the one kernel; checked once
         # against the logprob operator on the drawn ids before it is timed
         d_ids, d_pol = sampler.sample(logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
@@ -281,8 +288,10 @@ def lmhead_throughput(sampler, iters: int = 3):
         gbps = alg / (ms_small * 1e-3) / 1e9
         decode[f"n{rows}"] = {"ms": ms_small, "bit_identical_to_the_rows_of_the_large_call": True,
                               "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                                           "frac": gbps / HBM_PEAK_GBPS, "bytes_per_call": alg, "traffic": None,
-                                           "kernel": "lmhead_partials (units as work items) + lmhead_combine_units"}}
+                                           "frac": gbps / HBM_PEAK_GBPS, "bytes_per_call": alg,
+                                           **traffic_fields(f"lmhead_n{rows}"),
+                                           "kernel": ("lmhead_partials_narrow" if rows <= 128 else "lmhead_partials (units as "
+                                                      "work items)") + " + lmhead_combine_units"}}
     return {"config": "hidden bf16 [32768,4096] ~ N(0,1), W bf16 [128256,4096] ~ N(0,0.02^2), seed 0; logits never stored",
             "ms": ms, "tokens_per_s": n / (ms * 1e-3),
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": 2500.0, "unit": "TFLOP/s",
