@@ -35,7 +35,7 @@ BYTES_PER_TOKEN = 2 * V + 8 + 4
 # hex digits of the SHA-256 of those files (concatenated in that order) at the time of the counter runs.
 CSRC = REPO / "kernel-align_amd" / "csrc"
 _SAMPLING_SOURCES = ("ka_common.h", "ka_sampling_common.h", "ka_sampling_topk.h", "ka_sampling_dense.h", "ka_sampling_draw.h",
-                     "ka_sampling.hip")
+                     "ka_sampling_kernel.h", "ka_sampling.hip", "ka_sampling_half.hip")
 _LMHEAD_SOURCES = ("ka_common.h", "ka_lmhead.hip", "ka_lmhead_narrow.h")
 STATIC_TRAFFIC = {
     "logprob_rows": ((2 * 1026607.7 + 258.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",

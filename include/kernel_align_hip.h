@@ -171,10 +171,15 @@ int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, in
  * against the other: KA_SAMPLE_FLAG_GENERAL_PATH runs the general radix-select path even where a shorter route
  * applies; KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK keeps the top-k route on its block-wide selection and tail instead of the
  * short ones it takes for top_k <= 256 (bound from pooled maxima up to top_k = 64, from a radix descent above).  Ids
- * and log-probabilities do not depend on the flags.
+ * and log-probabilities do not depend on the flags.  KA_SAMPLE_FLAG_TWO_ROWS_PER_CU / KA_SAMPLE_FLAG_ONE_ROW_PER_CU: the
+ * short top-k route (scalar top_k <= 256, 16-byte aligned 16-bit rows of at most 131,072 entries) exists on 512 and on
+ * 1024 threads per row; the library takes 512, with two rows resident per CU, for batches of more rows than the device has
+ * CUs, and these flags force either where the row qualifies (both give the same ids and the same log-probability bits).
  */
 #define KA_SAMPLE_FLAG_GENERAL_PATH 1u
 #define KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK 2u
+#define KA_SAMPLE_FLAG_TWO_ROWS_PER_CU 4u
+#define KA_SAMPLE_FLAG_ONE_ROW_PER_CU 8u
 int ka_sample_ex(int dtype, const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
                  float temperature, const float *temperature_rows, int32_t top_k, const int32_t *top_k_rows,
                  float top_p, const float *top_p_rows, const float *uniforms, int64_t *out_ids,

@@ -20,9 +20,17 @@ __device__ unsigned long long ka_dbg_stamps[16 * 16 + 32];  // [wavefront][point
 #define KA_DBG_SET(i_, v_) do { } while (0)
 #endif
 
-constexpr int S_THREADS = 1024;
+// Threads of a workgroup (one row).  1024 is the ordinary build.  A second build of the top-k kernel with 512 lets two
+// workgroups share a CU, so that one row's selection runs under the other row's read; it is launched for batches of more
+// rows than the device has CUs.  Every integer decision is the same function of the row in both.
+#ifndef KA_SAMPLING_THREADS
+#define KA_SAMPLING_THREADS 1024
+#endif
+constexpr int S_THREADS = KA_SAMPLING_THREADS;
+static_assert(S_THREADS == 1024 || S_THREADS == 512, "the sampling kernels are written for 1024 or 512 threads");
 constexpr int S_WAVES = S_THREADS / kWave;
 constexpr int BINS = 2048;
+constexpr int BINS_PER_THREAD = BINS / S_THREADS;  // of a histogram that the block scans in one step
 constexpr int FIX_BITS = 40;
 
 // ---------------------------------------------------------------------------
@@ -261,16 +269,22 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, Shared &sh) {
 __device__ __forceinline__ uint32_t select_count_bin(Shared &sh, uint32_t nb, uint32_t rank, uint32_t *above,
                                                      uint32_t *count) {
     const int tid = threadIdx.x;
-    // thread t owns the bins 2t and 2t+1 counted from the top
-    const int rb0 = 2 * tid, rb1 = 2 * tid + 1;
-    const uint32_t c0 = rb0 < int(nb) ? sh.h.cnt[nb - 1 - rb0] : 0u;
-    const uint32_t c1 = rb1 < int(nb) ? sh.h.cnt[nb - 1 - rb1] : 0u;
+    // thread t owns the bins BINS_PER_THREAD * t + j counted from the top
+    uint32_t c[BINS_PER_THREAD], mine = 0;
+#pragma unroll
+    for (int j = 0; j < BINS_PER_THREAD; ++j) {
+        const int rb = BINS_PER_THREAD * tid + j;
+        c[j] = rb < int(nb) ? sh.h.cnt[nb - 1 - rb] : 0u;
+        mine += c[j];
+    }
     uint32_t total;
-    const uint32_t excl = block_excl_scan<uint32_t>(c0 + c1, sh.wave_u32, &total);
-    if (excl < rank && rank <= excl + c0) {
-        sh.sel_digit = nb - 1 - rb0; sh.sel_above = excl; sh.sel_count = c0;
-    } else if (excl + c0 < rank && rank <= excl + c0 + c1) {
-        sh.sel_digit = nb - 1 - rb1; sh.sel_above = excl + c0; sh.sel_count = c1;
+    uint32_t run = block_excl_scan<uint32_t>(mine, sh.wave_u32, &total);
+#pragma unroll
+    for (int j = 0; j < BINS_PER_THREAD; ++j) {
+        if (run < rank && rank <= run + c[j]) {
+            sh.sel_digit = nb - 1 - uint32_t(BINS_PER_THREAD * tid + j); sh.sel_above = run; sh.sel_count = c[j];
+        }
+        run += c[j];
     }
     __syncthreads();
     const uint32_t digit = sh.sel_digit;
@@ -297,18 +311,24 @@ __device__ __forceinline__ void clear_hist(Shared &sh) {
 constexpr float kLseLog2e = 1.44269504088896340736f;
 constexpr float kLseFloor = -1.0e30f;  // running maxima start here: (old max - new max) is never inf - inf
 
+// The fold is defined on 1024 lanes: lane t takes the vectors t, t + 1024, ... of the row.  A block of 512 threads lets
+// thread t stand in for the lanes t and t + 512 with an accumulator each, so both builds return the same bits.
+constexpr int LSE_LANES = 1024;
+constexpr int LSE_WAVES = LSE_LANES / kWave;
+constexpr int LSE_PER_THREAD = LSE_LANES / S_THREADS;
+
 struct PolicyLse {  // in LDS
-    float wave_ml2[S_WAVES];  // maximum * log2(e) of each wavefront's elements
-    float wave_s[S_WAVES];    // sum of 2^(x * log2(e) - wave_ml2)
+    float wave_ml2[LSE_WAVES];  // maximum * log2(e) of the elements of each wavefront of the 1024-lane order
+    float wave_s[LSE_WAVES];    // sum of 2^(x * log2(e) - wave_ml2)
     // log-probability of element `hit` of the row (thread 0, after a barrier behind to_block)
     template <typename T> __device__ __forceinline__ float finish(const typename T::raw_t *rp, int64_t hit, int vocab) const {
         if (hit < 0 || hit >= vocab) return __builtin_nanf("");
         float big = wave_ml2[0];
 #pragma unroll
-        for (int w = 1; w < S_WAVES; ++w) big = fmaxf(big, wave_ml2[w]);
+        for (int w = 1; w < LSE_WAVES; ++w) big = fmaxf(big, wave_ml2[w]);
         float total = 0.0f;
 #pragma unroll
-        for (int w = 0; w < S_WAVES; ++w) total += wave_s[w] * fast_exp2(wave_ml2[w] - big);
+        for (int w = 0; w < LSE_WAVES; ++w) total += wave_s[w] * fast_exp2(wave_ml2[w] - big);
         const double lse = (double(big) + log2(double(total))) * 0.693147180559945309417232;
         return float(double(T::widen(rp[hit])) - lse);
     }
@@ -339,16 +359,72 @@ struct LaneLse {
         m = mn;
         ml2 = ml2n;
     }
-    // every thread of the block calls this; a barrier must follow before PolicyLse::finish
-    __device__ __forceinline__ void to_block(PolicyLse &out) const {
+    // every thread of the block calls this; a barrier must follow before PolicyLse::finish.  `stand_in`: which of the
+    // thread's lanes of the 1024-lane order this accumulator belongs to (lane threadIdx.x + stand_in * S_THREADS).
+    __device__ __forceinline__ void to_block(PolicyLse &out, int stand_in = 0) const {
         const float wm = wave_max(ml2);
         const float ws = wave_sum(s * fast_exp2(ml2 - wm));
         if ((threadIdx.x & (kWave - 1)) == 0) {
-            out.wave_ml2[threadIdx.x / kWave] = wm;
-            out.wave_s[threadIdx.x / kWave] = ws;
+            out.wave_ml2[threadIdx.x / kWave + stand_in * S_WAVES] = wm;
+            out.wave_s[threadIdx.x / kWave + stand_in * S_WAVES] = ws;
         }
     }
 };
+
+// The accumulators of one thread: one per lane of the 1024-lane order it stands in for.
+struct ThreadLse {
+    LaneLse lane[LSE_PER_THREAD];
+    __device__ __forceinline__ void to_block(PolicyLse &out) const {
+#pragma unroll
+        for (int e = 0; e < LSE_PER_THREAD; ++e) lane[e].to_block(out, e);
+    }
+};
+
+// Largest element of a 16-byte vector.
+template <typename T> __device__ __forceinline__ float vector_max(const uint4 &q) {
+    const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
+    float vm = T::widen(e[0]);
+#pragma unroll
+    for (int j = 1; j < T::kPerVec; ++j) vm = fmaxf(vm, T::widen(e[j]));
+    return vm;
+}
+
+// Log-sum-exp partials of a whole row by the block, in the order the short top-k route folds a row while it reads it:
+// lane t of the 1024-lane order takes the vectors t, t + 1024, ... (one rescale per vector), then element t of the ragged
+// tail; an unaligned row goes element by element (t, t + 1024, ...).  The value is a function of the row alone.
+template <typename T>
+__device__ __forceinline__ void row_lse_to_block(const typename T::raw_t *rp, int vocab, bool vec, PolicyLse &out) {
+    constexpr int EPV = T::kPerVec;
+    ThreadLse acc;
+#pragma unroll
+    for (int e = 0; e < LSE_PER_THREAD; ++e) {
+        const int lane = int(threadIdx.x) + e * S_THREADS;
+        if (vec) {
+            const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
+            const int nvec = vocab / EPV;
+            constexpr int U = 4;  // loads in flight; the vectors are folded in their order
+            auto fold = [&](const uint4 &q) {
+                float x[EPV];
+                T::unpack(q, x);
+                acc.lane[e].add_vector(x, vector_max<T>(q));
+            };
+            int v = lane;
+            for (; v + (U - 1) * LSE_LANES < nvec; v += U * LSE_LANES) {
+                uint4 q[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) q[u] = vp[v + u * LSE_LANES];
+#pragma unroll
+                for (int u = 0; u < U; ++u) fold(q[u]);
+            }
+            for (; v < nvec; v += LSE_LANES) fold(vp[v]);
+            const int i = nvec * EPV + lane;
+            if (i < vocab) acc.lane[e].add(T::widen(rp[i]));
+        } else {
+            for (int i = lane; i < vocab; i += LSE_LANES) acc.lane[e].add(T::widen(rp[i]));
+        }
+    }
+    acc.to_block(out);
+}
 
 // ---------------------------------------------------------------------------
 // Row traversal: f(index, raw element) for every element, any order.

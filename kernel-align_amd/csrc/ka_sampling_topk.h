@@ -31,7 +31,10 @@ namespace {
 // ---------------------------------------------------------------------------
 constexpr int SHORT_TOPK = 256;      // largest top_k the short route serves
 constexpr int SHORT_POOL_TOPK = 64;  // up to here the bound comes from pooled group maxima, above from a radix descent
-constexpr int SHORT_GROUPS = 128;    // the 1024 lane maxima are pooled into this many group maxima (8 lanes each)
+constexpr int SHORT_GROUPS = 128;    // the lane maxima are pooled into this many group maxima (8 lanes each of 1024, 4 of 512)
+constexpr int SHORT_POOL = S_THREADS / SHORT_GROUPS;  // lanes per group
+constexpr int BLOCK_CAND = CAND_CAP < S_THREADS ? CAND_CAP : S_THREADS;  // candidates the block-wide tail ranks (one per thread)
+static_assert(SHORT_POOL == 8 || SHORT_POOL == 4, "the pooling below is written for groups of 8 or 4 lanes");
 constexpr int SHORT_VECS = 512;      // candidate vectors the short route takes (16 bytes each in LDS)
 constexpr int SHORT_CAND = 512;      // candidates its tail takes (eight per lane of one wavefront)
 
@@ -146,6 +149,8 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
                                          PolicyLse &lse) {
     const int tid = threadIdx.x;
     // top_k <= 64 takes the short route unless the caller asks for the block-wide one (the two give the same ids)
+    // (the build with 512 threads has no block-wide route: what its short route cannot take goes to the radix path)
+    if (S_THREADS != 1024 && (top_k > SHORT_TOPK || block_wide_only)) return 0;
     const bool short_route = top_k <= SHORT_TOPK && !block_wide_only;
     // 1. lane maxima of the raw values (float max: one convert and half a v_max3 per element; which of
     //    -0 / +0 it returns does not matter, any lower bound of the top_k-th element will do)
@@ -168,9 +173,10 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
     const int trk_need = (nvec + TRK_VECS * S_THREADS - 1) / (TRK_VECS * S_THREADS);
     const int trk_rounds = T::kBytes == 4 ? trk_need : 1;
     const bool tracked = vec && !resident && trk_need <= (T::kBytes == 4 ? 4 : 1);
-    // the short route folds the row's log-sum-exp while it reads the row (it never keeps the row in registers)
-    const bool take_lse = short_route && policy_slot != nullptr;
-    LaneLse acc_lse;
+    // the short route folds the row's log-sum-exp while it reads a row it tracks (the order of row_lse_to_block, so the
+    // value does not depend on the route); other rows get the fold's own pass at the end of the kernel
+    const bool take_lse = short_route && policy_slot != nullptr && tracked;
+    ThreadLse acc_lse;
     uint4 held[RES_VECS];
     // The slot maxima of a 16-bit row are kept in the row's own 16 bits, two per register (they are elements of the
     // row, so nothing is lost): 32 floats next to the loads in flight would spill.
@@ -197,13 +203,7 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
         return __uint_as_float(vstore[slot]);
     };
     float lmaxf = -__builtin_inff();
-    auto vector_max = [](const uint4 &q) {
-        const typename T::raw_t *e = reinterpret_cast<const typename T::raw_t *>(&q);
-        float vm = T::widen(e[0]);
-#pragma unroll
-        for (int j = 1; j < EPV; ++j) vm = fmaxf(vm, T::widen(e[j]));
-        return vm;
-    };
+    auto vector_max = [](const uint4 &q) { return ka::vector_max<T>(q); };
     if (tracked) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
 #pragma unroll 1
@@ -232,7 +232,7 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
                         if (take_lse) {
                             float x[EPV];
                             T::unpack(q[s], x);
-                            acc_lse.add_vector(x, vm);
+                            acc_lse.lane[(g * TRK_BATCH + s) % LSE_PER_THREAD].add_vector(x, vm);
                         }
                     }
                     set_slot_max(g * TRK_BATCH + s, vm, round == 0);
@@ -243,7 +243,7 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
         const int i = nvec * EPV + tid;  // ragged tail of the row
         if (i < vocab) {
             lmaxf = fmaxf(lmaxf, T::widen(rp[i]));
-            if (take_lse) acc_lse.add(T::widen(rp[i]));
+            if (take_lse) acc_lse.lane[0].add(T::widen(rp[i]));
         }
     } else if (resident) {
         const uint4 *vp = reinterpret_cast<const uint4 *>(rp);
@@ -265,7 +265,6 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
     } else {
         for_each_raw<T, 8>(rp, vocab, vec, [&](int, typename T::raw_t raw) {
             lmaxf = fmaxf(lmaxf, T::widen(raw));
-            if (take_lse) acc_lse.add(T::widen(raw));
         });
     }
     if (take_lse) acc_lse.to_block(lse);  // a barrier follows on every way on (pooling of the maxima, radix descent)
@@ -314,31 +313,32 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
         float gmax = lmaxf;
         gmax = fmaxf(gmax, __uint_as_float(dpp_xor1(__float_as_uint(gmax))));
         gmax = fmaxf(gmax, __uint_as_float(dpp_xor2(__float_as_uint(gmax))));
-        gmax = fmaxf(gmax, __uint_as_float(dpp_half_mirror(__float_as_uint(gmax))));
-        if ((tid & 7) == 0) sh.c.skey[tid >> 3] = __float_as_uint(gmax);
+        if (SHORT_POOL == 8) gmax = fmaxf(gmax, __uint_as_float(dpp_half_mirror(__float_as_uint(gmax))));
+        if ((tid & (SHORT_POOL - 1)) == 0) sh.c.skey[tid / SHORT_POOL] = __float_as_uint(gmax);
         if (tid == 0) { sh.n_cand = 0; sh.n_vec = 0; sh.hit = -1; sh.cand_kmax = 0; }
         __syncthreads();
         // S2. Eight threads rank one group maximum among the 128 (descending, ties by position): sixteen compares
         //     each, summed inside the group of eight lanes.  Exactly one maximum has rank top_k - 1.
         {
-            const int v = tid >> 3, part = tid & 7;
+            constexpr int SHARE = SHORT_GROUPS / SHORT_POOL;  // group maxima one thread compares against
+            const int v = tid / SHORT_POOL, part = tid & (SHORT_POOL - 1);
             const float x = __uint_as_float(sh.c.skey[v]);
-            const uint4 *others = reinterpret_cast<const uint4 *>(sh.c.skey + part * 16);
+            const uint4 *others = reinterpret_cast<const uint4 *>(sh.c.skey + part * SHARE);
             uint32_t cnt = 0;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int q = 0; q < SHARE / 4; ++q) {
                 const uint4 o = others[q];
                 const uint32_t ow[4] = {o.x, o.y, o.z, o.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float of = __uint_as_float(ow[e]);
-                    const int j = part * 16 + q * 4 + e;
+                    const int j = part * SHARE + q * 4 + e;
                     cnt += (of > x || (of == x && j < v)) ? 1u : 0u;
                 }
             }
             cnt += dpp_xor1(cnt);
             cnt += dpp_xor2(cnt);
-            cnt += dpp_half_mirror(cnt);
+            if (SHORT_POOL == 8) cnt += dpp_half_mirror(cnt);
             if (part == 0 && cnt == uint32_t(top_k - 1)) sh.max_key = __float_as_uint(x);
         }
         __syncthreads();
@@ -450,7 +450,7 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
                         }
                     }
                     uint32_t both = cnt | (cnt_i << 16);  // both counts stay below 2^16: one register through the DPP sums
-                    both += dpp_xor1(both);
+                    if (PARTS >= 2) both += dpp_xor1(both);
                     if (PARTS >= 4) both += dpp_xor2(both);
                     if (PARTS >= 8) both += dpp_half_mirror(both);
                     if (PARTS >= 16) both += dpp_row_mirror(both);
@@ -466,10 +466,10 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
                         by_index_idx(sh)[cnt_i] = ii;
                     }
                 };
-                if (nc <= 64u) rank_candidates(std::integral_constant<uint32_t, 16>{});
-                else if (nc <= 128u) rank_candidates(std::integral_constant<uint32_t, 8>{});
-                else if (nc <= 256u) rank_candidates(std::integral_constant<uint32_t, 4>{});
-                else rank_candidates(std::integral_constant<uint32_t, 2>{});
+                if (nc <= 64u) rank_candidates(std::integral_constant<uint32_t, S_THREADS / 64>{});
+                else if (nc <= 128u) rank_candidates(std::integral_constant<uint32_t, S_THREADS / 128>{});
+                else if (nc <= 256u) rank_candidates(std::integral_constant<uint32_t, S_THREADS / 256>{});
+                else rank_candidates(std::integral_constant<uint32_t, S_THREADS / 512>{});
                 __syncthreads();
                 KA_STAMP(5);   // candidates sorted
                 if (tid < kWave) {  // one wavefront finishes the row; the others are done
@@ -489,8 +489,10 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
                 }
                 return take_lse ? 2 : 1;
             }
+            if (S_THREADS != 1024) return 0;
             have_candidates = true;  // more than 512 candidates (a large tie group): the block-wide tail ranks them
         }
+        if (S_THREADS != 1024) return 0;
         __syncthreads();  // too many candidate vectors: the block-wide route starts over with its exact bound
     }
     if (!have_candidates) {
@@ -550,7 +552,7 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
     KA_STAMP(4);   // candidates collected
     }
     const uint32_t nc = sh.n_cand;
-    if (nc > CAND_CAP) return 0;
+    if (nc > BLOCK_CAND) return 0;
     // 3a. scale the candidates and rank them by (key desc, index asc)
     uint32_t my_key = 0, my_idx = 0;
     if (tid < int(nc)) {

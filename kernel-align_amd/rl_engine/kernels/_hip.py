@@ -64,6 +64,8 @@ SIGNATURES = {
 # Route selection flags of ka_sample_ex (verification only; results do not depend on them).
 SAMPLE_FLAG_GENERAL_PATH = 1
 SAMPLE_FLAG_BLOCK_WIDE_TOPK = 2
+SAMPLE_FLAG_TWO_ROWS_PER_CU = 4
+SAMPLE_FLAG_ONE_ROW_PER_CU = 8
 
 # Size of the static device array behind ka_lmhead_logprob_bf16_noalloc (KA_LMHEAD_STATIC_SCRATCH_BYTES).
 LMHEAD_STATIC_SCRATCH_BYTES = 16 << 20

@@ -79,7 +79,8 @@ def test_sampling_argument_checks():
     assert ex(0, None, 0, 128, 128, 1.0, None, 0, None, 1.0, None, None, None, None, None, 0, None, 0, None) == _hip.KA_OK
     assert ex(7, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG   # dtype code
     assert ex(0, p, 2, 128, 128, 0.0, None, 0, None, 1.0, None, p, p, None, None, 0, None, 0, None) == _hip.KA_ERR_BAD_ARG   # scalar T
-    assert ex(0, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 4, None, 0, None) == _hip.KA_ERR_BAD_ARG   # flag bits
+    assert ex(0, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 16, None, 0, None) == _hip.KA_ERR_BAD_ARG   # flag bits
+    assert ex(0, p, 2, 128, 128, 1.0, None, 0, None, 1.0, None, p, p, None, None, 12, None, 0, None) == _hip.KA_ERR_BAD_ARG   # both workgroup sizes
     assert b"flag" in lib.ka_last_error()
     # a per-row array replaces its scalar, which is then not checked: the call gets past the scalar checks and
     # is stopped by the next host check (stride < vocab), so nothing is ever launched on these made-up pointers

@@ -23,7 +23,9 @@ def run(sampler, logits, u, k, p, temp, route_flags=0):
                           route_flags=route_flags).cpu()
 
 
-ROUTES = (0, _hip.SAMPLE_FLAG_BLOCK_WIDE_TOPK, _hip.SAMPLE_FLAG_GENERAL_PATH)   # shortest, block-wide top-k, radix
+# shortest, block-wide top-k, radix; the short top-k route on 512 and on 1024 threads per row (where the row qualifies)
+ROUTES = (0, _hip.SAMPLE_FLAG_BLOCK_WIDE_TOPK, _hip.SAMPLE_FLAG_GENERAL_PATH, _hip.SAMPLE_FLAG_TWO_ROWS_PER_CU,
+          _hip.SAMPLE_FLAG_ONE_ROW_PER_CU)
 
 
 def check_exact(sampler, logits, u, k, p, temp):
@@ -221,9 +223,9 @@ def test_fast_and_radix_paths_are_the_same_function(sampler):
         cases.append((torch.zeros(4, 128256).to(dtype), 50, 0.3, 0.7))                                  # overflow -> radix
     for logits, k, p, temp in cases:
         u = torch.rand(logits.shape[0], generator=g)
-        fast, block, radix = (run(sampler, logits, u, k, p, temp, f) for f in ROUTES)
-        assert torch.equal(fast, radix) and torch.equal(fast, block)
-        assert torch.equal(fast, exact.sample(logits, temp, k, p, u))
+        want = exact.sample(logits, temp, k, p, u)
+        for f in ROUTES:
+            assert torch.equal(run(sampler, logits, u, k, p, temp, f), want), f"route_flags={f}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -261,7 +263,53 @@ def test_wavefront_route_of_small_top_k(sampler, dtype):
 def test_unknown_route_flag_is_refused(sampler):
     logits, u = cfg5_sampling(4, vocab=1000)
     with pytest.raises(ValueError, match="flag"):
-        sampler.sample(logits.cuda(), top_k=5, uniforms=u.cuda(), route_flags=8)
+        sampler.sample(logits.cuda(), top_k=5, uniforms=u.cuda(), route_flags=16)
+    with pytest.raises(ValueError, match="flag"):   # the two workgroup sizes exclude each other
+        sampler.sample(logits.cuda(), top_k=5, uniforms=u.cuda(),
+                       route_flags=_hip.SAMPLE_FLAG_TWO_ROWS_PER_CU | _hip.SAMPLE_FLAG_ONE_ROW_PER_CU)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("vocab", [128256, 131072, 4096, 1000])
+def test_two_rows_per_cu_build_returns_the_same_bits(sampler, dtype, vocab):
+    """The short top-k route on 512 threads per row (two rows resident per CU, what a batch of more rows than CUs gets)
+    against the same route on 1024 threads: ids, filtered log-probability and policy log-probability bit for bit, on
+    ordinary rows, a tie group of half the row, an all-equal row and a row with five numbers above -inf (the last three
+    leave the short route, in either build for its own reason); ids also against the exact oracle."""
+    g = torch.Generator().manual_seed(77)
+    batch = 12
+    logits = (torch.randn(batch, vocab, generator=g) * 3).to(dtype)
+    logits[0, : vocab // 2] = 1.5
+    logits[1] = 0.25
+    logits[2, 5:] = float("-inf")
+    u = torch.rand(batch, generator=g)
+    dev_logits, dev_u = logits.cuda(), u.cuda()
+    for k in (1, 50, 64, 65, 256):
+        for p, temp in ((None, 1.0), (0.9, 0.7), (0.3, 50.0)):
+            one = sampler.sample(dev_logits, top_k=k, top_p=p, temperature=temp, uniforms=dev_u, return_logprob=True,
+                                 return_policy_logprob=True, route_flags=_hip.SAMPLE_FLAG_ONE_ROW_PER_CU)
+            two = sampler.sample(dev_logits, top_k=k, top_p=p, temperature=temp, uniforms=dev_u, return_logprob=True,
+                                 return_policy_logprob=True, route_flags=_hip.SAMPLE_FLAG_TWO_ROWS_PER_CU)
+            assert torch.equal(one[0], two[0]), (k, p, temp)
+            assert torch.equal(one[1].view(torch.int32), two[1].view(torch.int32)), (k, p, temp)
+            assert torch.equal(one[2].view(torch.int32), two[2].view(torch.int32)), (k, p, temp)
+            assert torch.equal(two[0].cpu(), exact.sample(logits, temp, k, p, u)), (k, p, temp)
+
+
+def test_a_batch_of_more_rows_than_cus_matches_its_rows_sampled_in_small_batches(sampler):
+    """The library switches to two rows per CU above one row per CU: ids and both log-probabilities of a 600-row call are
+    those of the same rows in calls of 200."""
+    logits, u = cfg5_sampling(600)
+    dev_logits, dev_u = logits.cuda(), u.cuda()
+    big = sampler.sample(dev_logits, top_k=50, top_p=0.9, temperature=0.7, uniforms=dev_u, return_logprob=True,
+                         return_policy_logprob=True)
+    for lo in (0, 200, 400):
+        part = sampler.sample(dev_logits[lo:lo + 200], top_k=50, top_p=0.9, temperature=0.7, uniforms=dev_u[lo:lo + 200],
+                              return_logprob=True, return_policy_logprob=True)
+        for a, b in zip(big, part):
+            assert torch.equal(a[lo:lo + 200].view(torch.int32 if a.dtype == torch.float32 else a.dtype),
+                               b.view(torch.int32 if b.dtype == torch.float32 else b.dtype))
+    assert torch.equal(big[0].cpu(), exact.sample(logits, 0.7, 50, 0.9, u))
 
 
 def test_huge_temperature_folds_values_together(sampler):
