@@ -226,6 +226,25 @@ int ka_lmhead_logprob_entropy_bf16(const void *hidden, const void *weight, const
                                    void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /*
+ * ka_lmhead_logprob_bf16 that also returns every row's log-sum-exp over the vocabulary, lse[r] (fp32), which the
+ * backward below takes; same kernels, same workspace, same log-probabilities bit for bit.
+ *
+ * ka_lmhead_dlogits_bf16: the first half of the backward of ka_lmhead_logprob_bf16.  The logits tiles are computed
+ * again by the forward's MFMA kernel, and every logit x of row r goes out as
+ * dlogits[r, v] = grad_logprob[r] * ([v == ids[r]] - exp(x - lse[r])), rounded to bf16, into a [n_rows, vocab] matrix
+ * (row stride in elements, a multiple of 4, matrix 8-byte aligned); the logits themselves are never stored.  The
+ * caller contracts the matrix with weight (gradient of hidden) and with hidden (gradient of weight).  An id outside
+ * [0, vocab) contributes no one-hot term.  No workspace.  No counterpart in the reference, whose operators are
+ * inference-only (rl_engine/kernels/sampling.py:38,91).
+ */
+int ka_lmhead_logprob_lse_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out, float *lse,
+                               int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
+                               size_t workspace_bytes, void *hip_stream);
+int ka_lmhead_dlogits_bf16(const void *hidden, const void *weight, const int64_t *ids, const float *lse,
+                           const float *grad_logprob, void *dlogits, int64_t dlogits_row_stride, int64_t n_rows,
+                           int64_t hidden_dim, int64_t vocab, void *hip_stream);
+
+/*
  * ka_lmhead_logprob_bf16 for callers that cannot allocate device memory or bring a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same kernels, same results bit
  * for bit; the per-split partials go to a static array in device memory (KA_LMHEAD_STATIC_SCRATCH_BYTES,

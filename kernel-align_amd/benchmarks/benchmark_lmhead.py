@@ -80,9 +80,27 @@ def main() -> int:
         grad = torch.randn(args.rows, generator=g, device="cuda")
         torch.cuda.reset_peak_memory_stats()
         before = torch.cuda.memory_allocated()
+        # the gradient matrix of a chunk from the library GEMM + the two logprob kernels (the default) ...
         ms_b = timed(lambda: sampler.fused_linear_logp_backward(hidden, weight, ids, grad), max(2, args.iters // 2), warmup=1)
         out.update({"backward_ms": ms_b, "backward_tflops": 3.0 * flop / ms_b / 1e9,
                     "backward_peak_extra_bytes": torch.cuda.max_memory_allocated() - before})
+        # ... and from the forward's kernel with the softmax gradient as its epilogue (lse= option)
+        _, lse = sampler.fused_linear_logp(hidden, weight, ids, return_lse=True)
+        ms_f = timed(lambda: sampler.fused_linear_logp_backward(hidden, weight, ids, grad, lse=lse), max(2, args.iters // 2), warmup=1)
+        out.update({"backward_with_dlogits_kernel_ms": ms_f})
+        chunk_rows = min(args.rows, 8192)
+        dl = torch.empty(chunk_rows, args.vocab, dtype=torch.bfloat16, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+        def front_fused():
+            assert sampler._lib.ka_lmhead_dlogits_bf16(hidden.data_ptr(), weight.data_ptr(), ids.data_ptr(), lse.data_ptr(),
+                                                       grad.data_ptr(), dl.data_ptr(), args.vocab, chunk_rows, args.hidden,
+                                                       args.vocab, stream) == 0
+        def front_gemm():
+            logits = torch.matmul(hidden[:chunk_rows], weight.t())
+            logp = sampler.compute_logp(logits, ids[:chunk_rows])
+            sampler.compute_logp_backward(logits, ids[:chunk_rows], logp, grad[:chunk_rows], inplace=True)
+        out.update({"front_half_rows": chunk_rows, "front_half_dlogits_kernel_ms": timed(front_fused, args.iters),
+                    "front_half_gemm_and_logprob_kernels_ms": timed(front_gemm, args.iters)})
     print(json.dumps(out))
     return 0
 

@@ -211,11 +211,22 @@ typedef __attribute__((address_space(3))) void lds_void;
 // 64-bit offsets; the ordinary kernel keeps 32-bit offsets from the two base pointers, which is 1 - 2 % faster.
 // ENTROPY: also accumulate sum(x * exp(x - max)) per token (one more FMA per logit), from which the fold derives the
 // entropy of the row's softmax; it goes out in the fourth field of the partial.
-template <bool WIDE, bool ENTROPY>
+// DLOGITS: the backward's first half instead of the forward.  The same tiles are computed, but each logit x of token n
+// goes out as the gradient of that token's log-probability with respect to it, grad[n] * ([v == id_n] - exp(x - lse[n])),
+// rounded to bf16, into a [n_rows, vocab] matrix; lse[n] is the row's log-sum-exp as the forward returns it.  No partials,
+// no folds; items are (token block, split) pairs.
+struct DlogitsArgs {
+    const float *lse;    // [n_rows]
+    const float *grad;   // [n_rows] upstream gradient of the log-probabilities
+    uint16_t *out;       // [n_rows, row_stride] bf16
+    int64_t row_stride;  // elements, a multiple of 4 (8-byte stores)
+};
+
+template <bool WIDE, bool ENTROPY, bool DLOGITS = false>
 __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     const uint16_t *__restrict__ hidden, const uint16_t *__restrict__ weight, const int64_t *__restrict__ ids,
     Partial *__restrict__ partials, int n_rows, int hdim, int vocab, int n_token_blocks,
-    SplitPlan plan, int n_virtual, int fine) {
+    SplitPlan plan, int n_virtual, int fine, DlogitsArgs dl) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];  // [stage][A = W slab | B = hidden slab]
 
     const int tid = threadIdx.x;
@@ -239,6 +250,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
     float m_run[4], ml2_run[4], s_run[4], xt[4];  // ml2_run = m_run * log2(e), kept so that it is never recomputed
     float a_run[4];                               // ENTROPY: sum of x * exp(x - m_run)
     int target[4];
+    float lse2[4], gup[4];                        // DLOGITS: lse * log2(e) and the upstream gradient of the lane's tokens
 
     // Global -> LDS copies.  One global_load_lds_dwordx4 moves 16 B per lane to LDS base + 16 * lane,
     // i.e. one wavefront fills eight consecutive 128-byte rows (eight full cache lines); instruction j of
@@ -384,7 +396,11 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         int64_t id = -1;
         if (n < n_rows) id = ids[n];
         target[tn] = (id >= 0 && id < vocab) ? int(id) : -1;
-        if (!fine && folder) {  // the split's running partial starts empty
+        if constexpr (DLOGITS) {
+            lse2[tn] = n < n_rows ? dl.lse[n] * kLog2e : 0.0f;
+            gup[tn] = n < n_rows ? dl.grad[n] : 0.0f;
+        }
+        if (!DLOGITS && !fine && folder) {  // the split's running partial starts empty
             float *p = split_acc + ((wave_n * 4 + tn) * 32 + l32) * 4;
             p[0] = kFloor;
             p[1] = 0.0f;
@@ -479,6 +495,35 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             const int d = target[tn] - (vt * LM_BM + wave_m * 128);
             const bool mine = d >= 0 && d < 128 && ((d >> 2) & 1) == lhalf;
             const int want = mine ? (((d >> 5) << 4) | ((d & 31) >> 3 << 2) | (d & 3)) : -1;  // tm*16 + r
+            if constexpr (DLOGITS) {
+                // four consecutive vocabulary rows of one token per store: 8 bytes at out[n, vrow0 + tm*32 + q*8 ..]
+                const int n = tok0 + wave_n * 128 + tn * 32 + l32;
+                uint16_t *const orow = dl.out + size_t(n < n_rows ? n : 0) * size_t(dl.row_stride) + vrow0;
+                const float g = gup[tn], l2 = lse2[tn];
+#pragma unroll
+                for (int tm = 0; tm < 4; ++tm)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        union { __bf16 h[4]; uint2 u; } pk;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float pr = fast_exp2(fmaf(acc[tm][tn][q * 4 + j], kLog2e, -l2));
+                            const float onehot = want == tm * 16 + q * 4 + j ? g : 0.0f;
+                            pk.h[j] = (__bf16)fmaf(-g, pr, onehot);
+                        }
+                        const int off = tm * 32 + q * 8;
+                        if (n < n_rows) {
+                            if (off + 3 < limit) {
+                                *reinterpret_cast<uint2 *>(orow + off) = pk.u;
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    if (off + j < limit) orow[off + j] = reinterpret_cast<const uint16_t *>(pk.h)[j];
+                            }
+                        }
+                    }
+                continue;
+            }
             float mn = m_run[tn];
             float part[4], parta[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             // Wavefront-uniform choice: almost every tile lies inside the vocabulary and holds no lane's target,
@@ -556,6 +601,7 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    if constexpr (!DLOGITS) {
     // ---- fold the two lane halves (rows 4..7 of each 8-row group live in lanes 32..63) ----
 #pragma unroll
     for (int tn = 0; tn < 4; ++tn) {
@@ -624,8 +670,9 @@ __global__ __launch_bounds__(LM_THREADS, 1) void lmhead_partials(
             }
         }
     }
+    }  // !DLOGITS
     }  // units
-    if (!fine && folder) {
+    if (!DLOGITS && !fine && folder) {
 #pragma unroll
         for (int tn = 0; tn < 4; ++tn) {
             const float *q = split_acc + ((wave_n * 4 + tn) * 32 + l32) * 4;
@@ -657,7 +704,8 @@ namespace {
 // The fold of a row's split partials, in split order, and the two results.  get(sp) returns the partial of split sp.
 // Written out operation by operation (no contraction): whoever produced the split partials, the bits are the same.
 template <typename Get>
-__device__ __forceinline__ void lm_finish_row(Get get, int n_splits, int64_t id, int vocab, float *out_slot, float *entropy_slot) {
+__device__ __forceinline__ void lm_finish_row(Get get, int n_splits, int64_t id, int vocab, float *out_slot, float *entropy_slot,
+                                              float *lse_slot) {
 #pragma clang fp contract(off)
     float mm = kFloor;
     for (int sp = 0; sp < n_splits; ++sp) mm = fmaxf(mm, get(sp).m);
@@ -672,6 +720,7 @@ __device__ __forceinline__ void lm_finish_row(Get get, int n_splits, int64_t id,
     }
     const double lse = double(mm) + log2(double(s)) * kLn2;
     if (entropy_slot != nullptr) *entropy_slot = float(lse - double(a) / double(s));  // -sum p log p = lse - sum p x
+    if (lse_slot != nullptr) *lse_slot = float(lse);
     if (id < 0 || id >= vocab) {
         *out_slot = __builtin_nanf("");
         return;
@@ -682,11 +731,12 @@ __device__ __forceinline__ void lm_finish_row(Get get, int n_splits, int64_t id,
 // One thread per row; the kernel before it has folded the units of every split.
 __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict__ partials,
                                                       const int64_t *__restrict__ ids, float *__restrict__ out,
-                                                      float *__restrict__ entropy, int n_rows, int vocab, int n_splits) {
+                                                      float *__restrict__ entropy, float *__restrict__ lse, int n_rows,
+                                                      int vocab, int n_splits) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= n_rows) return;
     lm_finish_row([&](int sp) { return partials[size_t(sp) * n_rows + n]; }, n_splits, ids[n], vocab, out + n,
-                  entropy != nullptr ? entropy + n : nullptr);
+                  entropy != nullptr ? entropy + n : nullptr, lse != nullptr ? lse + n : nullptr);
 }
 
 // Few rows: the kernel before it has written one partial per unit.  One wavefront per row: lane l folds the units of
@@ -695,8 +745,8 @@ __global__ __launch_bounds__(256) void lmhead_combine(const Partial *__restrict_
 constexpr int LM_FINE_MAX_SPLITS = 256;
 __global__ __launch_bounds__(256) void lmhead_combine_units(const Partial *__restrict__ partials,
                                                             const int64_t *__restrict__ ids, float *__restrict__ out,
-                                                            float *__restrict__ entropy, int n_rows, int vocab,
-                                                            SplitPlan plan) {
+                                                            float *__restrict__ entropy, float *__restrict__ lse,
+                                                            int n_rows, int vocab, SplitPlan plan) {
     __shared__ Partial folded[4][LM_FINE_MAX_SPLITS];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int n = blockIdx.x * 4 + wave;
@@ -722,7 +772,7 @@ __global__ __launch_bounds__(256) void lmhead_combine_units(const Partial *__res
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (lane == 0)
         lm_finish_row([&](int sp) { return folded[wave][sp]; }, n_splits, ids[n], vocab, out + n,
-                      entropy != nullptr ? entropy + n : nullptr);
+                      entropy != nullptr ? entropy + n : nullptr, lse != nullptr ? lse + n : nullptr);
 }
 
 inline int splits_for(int64_t vocab) {
@@ -786,11 +836,13 @@ int lm_current_device(bool need_scratch, LmDevice &out) {
         rc = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
         if (rc != hipSuccess) return check_hip(rc, "lmhead: querying the CU count");
         // the attribute belongs to the device, so it is set once per device and not once per process
-        const void *kernels[4] = {reinterpret_cast<const void *>(lmhead_partials<false, false>),
+        const void *kernels[6] = {reinterpret_cast<const void *>(lmhead_partials<false, false>),
                                   reinterpret_cast<const void *>(lmhead_partials<true, false>),
                                   reinterpret_cast<const void *>(lmhead_partials<false, true>),
-                                  reinterpret_cast<const void *>(lmhead_partials<true, true>)};
-        for (int k = 0; k < 4 && rc == hipSuccess; ++k)
+                                  reinterpret_cast<const void *>(lmhead_partials<true, true>),
+                                  reinterpret_cast<const void *>(lmhead_partials<false, false, true>),
+                                  reinterpret_cast<const void *>(lmhead_partials<true, false, true>)};
+        for (int k = 0; k < 6 && rc == hipSuccess; ++k)
             rc = hipFuncSetAttribute(kernels[k], hipFuncAttributeMaxDynamicSharedMemorySize, LM_LDS_BYTES);
         if (rc == hipSuccess)
             rc = hipFuncSetAttribute(reinterpret_cast<const void *>(lmhead_partials_narrow<1, false>),
@@ -837,7 +889,7 @@ int lm_check_args(const void *hidden, const void *weight, const int64_t *ids, co
 
 // Enqueues the two kernels; `partials` holds ka_lmhead_workspace_bytes(n_rows, ., vocab) bytes of device memory.
 int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const int64_t *ids, float *out,
-              float *entropy, int64_t n_rows, int64_t hidden_dim, int64_t vocab, Partial *partials, hipStream_t stream) {
+              float *entropy, float *lse, int64_t n_rows, int64_t hidden_dim, int64_t vocab, Partial *partials, hipStream_t stream) {
     const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
     const int n_splits = splits_for(vocab);
     const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
@@ -871,13 +923,13 @@ int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const
         const int rcn = check_hip(hipGetLastError(), "lmhead partials launch (few rows)");
         if (rcn != KA_OK) return rcn;
         hipLaunchKernelGGL(lmhead_combine_units, dim3(unsigned((n_rows + 3) / 4)), dim3(256), 0, stream, partials, ids,
-                           out, entropy, int(n_rows), int(vocab), plan);
+                           out, entropy, lse, int(n_rows), int(vocab), plan);
         return check_hip(hipGetLastError(), "lmhead combine launch");
     }
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, stream,
                            static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids, partials,
-                           int(n_rows), int(hidden_dim), int(vocab), n_token_blocks, plan, int(n_virtual), fine);
+                           int(n_rows), int(hidden_dim), int(vocab), n_token_blocks, plan, int(n_virtual), fine, DlogitsArgs{});
     };
     if (entropy != nullptr) {
         if (wide) launch(lmhead_partials<true, true>);
@@ -890,15 +942,15 @@ int lm_launch(const LmDevice &dev, const void *hidden, const void *weight, const
     if (rc != KA_OK) return rc;
     if (fine)
         hipLaunchKernelGGL(lmhead_combine_units, dim3(unsigned((n_rows + 3) / 4)), dim3(256), 0, stream, partials, ids,
-                           out, entropy, int(n_rows), int(vocab), plan);
+                           out, entropy, lse, int(n_rows), int(vocab), plan);
     else
         hipLaunchKernelGGL(lmhead_combine, dim3(unsigned((n_rows + 255) / 256)), dim3(256), 0, stream, partials, ids,
-                           out, entropy, int(n_rows), int(vocab), n_splits);
+                           out, entropy, lse, int(n_rows), int(vocab), n_splits);
     return check_hip(hipGetLastError(), "lmhead combine launch");
 }
 
 // Everything the workspace entry points share.
-int lm_with_workspace(const void *hidden, const void *weight, const int64_t *ids, float *out, float *entropy,
+int lm_with_workspace(const void *hidden, const void *weight, const int64_t *ids, float *out, float *entropy, float *lse,
                       int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace, size_t workspace_bytes,
                       void *hip_stream) {
     if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead: n_rows %lld < 0", (long long)n_rows);
@@ -911,7 +963,7 @@ int lm_with_workspace(const void *hidden, const void *weight, const int64_t *ids
     LmDevice dev;
     rc = lm_current_device(false, dev);
     if (rc != KA_OK) return rc;
-    return lm_launch(dev, hidden, weight, ids, out, entropy, n_rows, hidden_dim, vocab, static_cast<Partial *>(workspace),
+    return lm_launch(dev, hidden, weight, ids, out, entropy, lse, n_rows, hidden_dim, vocab, static_cast<Partial *>(workspace),
                      static_cast<hipStream_t>(hip_stream));
 }
 
@@ -921,7 +973,7 @@ int lm_with_workspace(const void *hidden, const void *weight, const int64_t *ids
 KA_EXPORT int ka_lmhead_logprob_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
                                      int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
                                      size_t workspace_bytes, void *hip_stream) {
-    return ka::lm_with_workspace(hidden, weight, ids, out, nullptr, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
+    return ka::lm_with_workspace(hidden, weight, ids, out, nullptr, nullptr, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
                                  hip_stream);
 }
 
@@ -929,8 +981,52 @@ KA_EXPORT int ka_lmhead_logprob_entropy_bf16(const void *hidden, const void *wei
                                              float *entropy, int64_t n_rows, int64_t hidden_dim, int64_t vocab,
                                              void *workspace, size_t workspace_bytes, void *hip_stream) {
     if (entropy == nullptr && n_rows > 0) return ka::fail(KA_ERR_BAD_ARG, "lmhead: null entropy pointer");
-    return ka::lm_with_workspace(hidden, weight, ids, out, entropy, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
+    return ka::lm_with_workspace(hidden, weight, ids, out, entropy, nullptr, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
                                  hip_stream);
+}
+
+KA_EXPORT int ka_lmhead_logprob_lse_bf16(const void *hidden, const void *weight, const int64_t *ids, float *out,
+                                         float *lse, int64_t n_rows, int64_t hidden_dim, int64_t vocab, void *workspace,
+                                         size_t workspace_bytes, void *hip_stream) {
+    if (lse == nullptr && n_rows > 0) return ka::fail(KA_ERR_BAD_ARG, "lmhead: null lse pointer");
+    return ka::lm_with_workspace(hidden, weight, ids, out, nullptr, lse, n_rows, hidden_dim, vocab, workspace, workspace_bytes,
+                                 hip_stream);
+}
+
+KA_EXPORT int ka_lmhead_dlogits_bf16(const void *hidden, const void *weight, const int64_t *ids, const float *lse,
+                                     const float *grad_logprob, void *dlogits, int64_t dlogits_row_stride, int64_t n_rows,
+                                     int64_t hidden_dim, int64_t vocab, void *hip_stream) {
+    using namespace ka;
+    if (n_rows < 0) return fail(KA_ERR_BAD_ARG, "lmhead dlogits: n_rows %lld < 0", (long long)n_rows);
+    if (n_rows == 0) return KA_OK;
+    if (lse == nullptr || grad_logprob == nullptr || dlogits == nullptr)
+        return fail(KA_ERR_BAD_ARG, "lmhead dlogits: null lse / grad_logprob / dlogits pointer");
+    int rc = lm_check_args(hidden, weight, ids, lse, n_rows, hidden_dim, vocab);
+    if (rc != KA_OK) return rc;
+    if (dlogits_row_stride < vocab || dlogits_row_stride % 4 != 0 || reinterpret_cast<uintptr_t>(dlogits) % 8 != 0)
+        return fail(KA_ERR_BAD_ARG, "lmhead dlogits: the gradient matrix must be 8-byte aligned with a row stride >= vocab that "
+                                    "is a multiple of 4 (got %lld)", (long long)dlogits_row_stride);
+    LmDevice dev;
+    rc = lm_current_device(false, dev);
+    if (rc != KA_OK) return rc;
+    const int n_vtiles = int((vocab + LM_BM - 1) / LM_BM);
+    const SplitPlan plan(n_vtiles, splits_for(vocab));
+    const int n_token_blocks = int((n_rows + LM_BN - 1) / LM_BN);
+    const int64_t n_virtual = ItemOrder(n_token_blocks, plan, 0).n_virtual();
+    if (n_virtual >= (int64_t(1) << 30)) return fail(KA_ERR_UNSUPPORTED, "lmhead dlogits: too many work items");
+    const int64_t resident = dev.cus >= LM_RESIDENT ? LM_RESIDENT : (dev.cus >= 8 ? dev.cus / 8 * 8 : 8);
+    const int64_t grid = n_virtual < resident ? n_virtual : resident;
+    const bool wide = n_rows * hidden_dim * 2 >= (int64_t(1) << 32) || vocab * hidden_dim * 2 >= (int64_t(1) << 32);
+    const DlogitsArgs dl{lse, grad_logprob, static_cast<uint16_t *>(dlogits), dlogits_row_stride};
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(unsigned(grid)), dim3(LM_THREADS), LM_LDS_BYTES, static_cast<hipStream_t>(hip_stream),
+                           static_cast<const uint16_t *>(hidden), static_cast<const uint16_t *>(weight), ids,
+                           static_cast<Partial *>(nullptr), int(n_rows), int(hidden_dim), int(vocab), n_token_blocks, plan,
+                           int(n_virtual), 0, dl);
+    };
+    if (wide) launch(lmhead_partials<true, false, true>);
+    else launch(lmhead_partials<false, false, true>);
+    return check_hip(hipGetLastError(), "lmhead dlogits launch");
 }
 
 KA_EXPORT int ka_lmhead_logprob_bf16_noalloc(const void *hidden, const void *weight, const int64_t *ids, float *out,
@@ -950,6 +1046,6 @@ KA_EXPORT int ka_lmhead_logprob_bf16_noalloc(const void *hidden, const void *wei
     rc = lm_current_device(true, dev);
     if (rc != KA_OK) return rc;
     // Nothing in the scratch has to start at zero: every partial the fold reads is written by this call's first kernel.
-    return lm_launch(dev, hidden, weight, ids, out, nullptr, n_rows, hidden_dim, vocab, static_cast<Partial *>(dev.scratch),
+    return lm_launch(dev, hidden, weight, ids, out, nullptr, nullptr, n_rows, hidden_dim, vocab, static_cast<Partial *>(dev.scratch),
                      static_cast<hipStream_t>(hip_stream));
 }

@@ -55,6 +55,10 @@ SIGNATURES = {
     "ka_lmhead_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "ka_lmhead_logprob_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                        c_void_p, c_size_t, c_void_p]),
+    "ka_lmhead_logprob_lse_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                           c_int64, c_void_p, c_size_t, c_void_p]),
+    "ka_lmhead_dlogits_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                                       c_int64, c_int64, c_void_p]),
     "ka_lmhead_logprob_entropy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                                                c_int64, c_void_p, c_size_t, c_void_p]),
     "ka_lmhead_logprob_bf16_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,

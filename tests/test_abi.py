@@ -115,6 +115,19 @@ def test_lmhead_argument_checks_and_workspace_size():
     assert ent(None, None, None, None, None, 0, 4096, 128256, None, 0, None) == _hip.KA_OK
     assert ent(p, p, p, p, None, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG           # entropy missing
     assert ent(p, p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 * 4 - 1, None) == _hip.KA_ERR_WORKSPACE
+    # the forward that also returns the log-sum-exp, and the backward's first half that takes it
+    with_lse = lib.ka_lmhead_logprob_lse_bf16
+    assert with_lse(None, None, None, None, None, 0, 4096, 128256, None, 0, None) == _hip.KA_OK
+    assert with_lse(p, p, p, p, None, 4, 4096, 128256, p, 1 << 20, None) == _hip.KA_ERR_BAD_ARG       # lse missing
+    assert with_lse(p, p, p, p, p, 4, 4096, 128256, p, 4 * 16 * 64 * 4 - 1, None) == _hip.KA_ERR_WORKSPACE
+    dl = lib.ka_lmhead_dlogits_bf16
+    assert dl(None, None, None, None, None, None, 0, 0, 4096, 128256, None) == _hip.KA_OK           # no rows
+    assert dl(p, p, p, p, p, p, 128256, -1, 4096, 128256, None) == _hip.KA_ERR_BAD_ARG
+    assert dl(p, p, p, None, p, p, 128256, 4, 4096, 128256, None) == _hip.KA_ERR_BAD_ARG            # lse missing
+    assert dl(p, p, p, p, p, p, 128255, 4, 4096, 128256, None) == _hip.KA_ERR_BAD_ARG               # stride < vocab
+    assert dl(p, p, p, p, p, p, 128258, 4, 4096, 128256, None) == _hip.KA_ERR_BAD_ARG               # stride % 4
+    assert dl(p, p, p, p, p, ctypes.c_void_p(4100), 128256, 4, 4096, 128256, None) == _hip.KA_ERR_BAD_ARG   # 8-byte alignment
+    assert dl(p, p, p, p, p, p, 128256, 4, 100, 128256, None) == _hip.KA_ERR_UNSUPPORTED            # H % 64
     # the variant without a workspace argument: same checks, and a size limit instead of a workspace check
     na = lib.ka_lmhead_logprob_bf16_noalloc
     assert na(None, None, None, None, 0, 4096, 128256, None) == _hip.KA_OK

@@ -53,6 +53,39 @@ def test_linear_logp_backward(sampler, n, h, v, chunk):
     assert torch.allclose(lp.detach().cpu(), O.lmhead_logprob_ref(hidden, weight, ids), atol=2e-2, rtol=0)
 
 
+@pytest.mark.parametrize("n,h,v", [(300, 256, 1000), (513, 128, 4100), (40, 64, 256)])
+def test_dlogits_kernel_against_the_closed_form(sampler, n, h, v):
+    """The backward's first half from the forward's MFMA kernel: lse of the forward against fp64, the gradient matrix
+    g * (onehot - softmax) against the fp64 closed form on fp64 logits (bf16 rounding of the result: relative 2^-8),
+    entries beyond the vocabulary of a padded row untouched, and the full backward through it tighter than through the
+    GEMM path (its logits are never rounded to bf16)."""
+    g = torch.Generator().manual_seed(n * 7 + v)
+    hidden = torch.randn(n, h, generator=g).bfloat16()
+    weight = (torch.randn(v, h, generator=g) * 0.05).bfloat16()
+    ids = torch.randint(0, v, (n,), generator=g)
+    w = torch.randn(n, generator=g)
+    hd, wd, idd, gd = hidden.cuda(), weight.cuda(), ids.cuda(), w.cuda()
+    logp, lse = sampler.fused_linear_logp(hd, wd, idd, return_lse=True)
+    assert torch.equal(logp, sampler.fused_linear_logp(hd, wd, idd))
+    logits64 = hidden.double() @ weight.double().t()
+    assert (lse.double().cpu() - torch.logsumexp(logits64, -1)).abs().max().item() < 1e-4
+    stride = v + 8
+    dl = torch.full((n, stride), 7.0, dtype=torch.bfloat16, device="cuda")
+    from rl_engine.kernels import _hip
+    _hip.check(sampler._lib.ka_lmhead_dlogits_bf16(hd.data_ptr(), wd.data_ptr(), idd.data_ptr(), lse.data_ptr(),
+                                                   gd.data_ptr(), dl.data_ptr(), stride, n, h, v,
+                                                   torch.cuda.current_stream().cuda_stream), "ka_lmhead_dlogits_bf16")
+    want = O.logprob_backward_closed_form(logits64, ids, w)
+    got = dl[:, :v].double().cpu()
+    assert ((got - want).abs() <= 2.0 ** -8 * want.abs() + 1e-6).all()
+    assert (dl[:, v:] == 7.0).all()
+    dh, dw = sampler.fused_linear_logp_backward(hd, wd, idd, gd, chunk_tokens=128, lse=lse)
+    dh_ref, dw_ref = O.lmhead_logprob_backward_ref(hidden, weight, ids, w)
+    assert rel_err(dh, dh_ref) < 1e-2 and rel_err(dw, dw_ref) < 1e-2
+    dh_g, dw_g = sampler.fused_linear_logp_backward(hd, wd, idd, gd, chunk_tokens=128)
+    assert rel_err(dh, dh_g.double().cpu()) < 2e-2 and rel_err(dw, dw_g.double().cpu()) < 2e-2
+
+
 def test_chunked_backward_direct_call_and_shapes(sampler):
     g = torch.Generator().manual_seed(5)
     hidden = torch.randn(2, 40, 192, generator=g).bfloat16().cuda()
