@@ -86,6 +86,29 @@ def test_dlogits_kernel_against_the_closed_form(sampler, n, h, v):
     assert rel_err(dh, dh_g.double().cpu()) < 2e-2 and rel_err(dw, dw_g.double().cpu()) < 2e-2
 
 
+def test_backward_holds_one_chunk_of_the_gradient_matrix(sampler):
+    """Peak device memory of the backward beyond its two results: one [chunk, V] bf16 matrix (plus the small per-row
+    vectors), whatever the number of rows - with either first half."""
+    g = torch.Generator(device="cuda").manual_seed(9)
+    n, h, v, chunk = 4096, 256, 32000, 512
+    hidden = torch.randn(n, h, generator=g, device="cuda").bfloat16()
+    weight = (torch.randn(v, h, generator=g, device="cuda") * 0.05).bfloat16()
+    ids = torch.randint(0, v, (n,), generator=g, device="cuda")
+    grad = torch.randn(n, generator=g, device="cuda")
+    _, lse = sampler.fused_linear_logp(hidden, weight, ids, return_lse=True)
+    for kw in ({}, {"lse": lse}):
+        sampler.fused_linear_logp_backward(hidden, weight, ids, grad, chunk_tokens=chunk, **kw)   # warm: library workspaces
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        dh, dw = sampler.fused_linear_logp_backward(hidden, weight, ids, grad, chunk_tokens=chunk, **kw)
+        torch.cuda.synchronize()
+        extra = torch.cuda.max_memory_allocated() - before
+        results = dh.numel() * 2 + dw.numel() * 4
+        one_chunk = chunk * v * 2
+        assert extra <= results + one_chunk + (4 << 20), (extra, results, one_chunk)
+
+
 def test_chunked_backward_direct_call_and_shapes(sampler):
     g = torch.Generator().manual_seed(5)
     hidden = torch.randn(2, 40, 192, generator=g).bfloat16().cuda()
