@@ -115,6 +115,19 @@ def test_weight_matrix_above_4_gib(sampler):
     assert (got - unfused).abs().max().item() <= TOL
     want = O.lmhead_logprob_ref(hidden[:8].cpu(), weight.cpu(), ids[:8].cpu(), dtype=torch.float32)
     assert (got[:8].cpu() - want).abs().max().item() <= TOL
+    # the backward's gradient matrix from the same (wide-addressing) kernel against the unfused logits on the GPU
+    got2, lse = sampler.fused_linear_logp(hidden, weight, ids, return_lse=True)
+    assert torch.equal(got2, got)
+    assert (lse - torch.logsumexp(logits, -1)).abs().max().item() <= TOL
+    grad = torch.randn(n, generator=g, device="cuda")
+    dl = torch.empty(n, vocab, dtype=torch.bfloat16, device="cuda")
+    from rl_engine.kernels import _hip
+    _hip.check(sampler._lib.ka_lmhead_dlogits_bf16(hidden.data_ptr(), weight.data_ptr(), ids.data_ptr(), lse.data_ptr(),
+                                                   grad.data_ptr(), dl.data_ptr(), vocab, n, hdim, vocab,
+                                                   torch.cuda.current_stream().cuda_stream), "ka_lmhead_dlogits_bf16")
+    want_dl = -torch.softmax(logits, -1) * grad[:, None]
+    want_dl[torch.arange(n, device="cuda"), ids] += grad
+    assert ((dl.float() - want_dl).abs() <= 2.0 ** -7 * want_dl.abs() + 1e-6).all()
 
 
 def test_leading_dims_and_invalid_ids(sampler):
