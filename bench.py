@@ -38,9 +38,9 @@ _SAMPLING_SOURCES = ("ka_common.h", "ka_sampling_common.h", "ka_sampling_topk.h"
                      "ka_sampling_kernel.h", "ka_sampling.hip", "ka_sampling_half.hip")
 _LMHEAD_SOURCES = ("ka_common.h", "ka_lmhead.hip", "ka_lmhead_narrow.h")
 STATIC_TRAFFIC = {
-    "logprob_rows": ((2 * 1026607.7 + 258.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",
+    "logprob_rows": ((2 * 4106340 + 1054.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",           # 32768 rows
                      ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
-    "logprob_backward_rows": ((2 * 1027116 + 2052133) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",
+    "logprob_backward_rows": ((2 * 4108350 + 8208390) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",  # 32768 rows
                               ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
     "sample_rows": ((2 * 32856.4 + 10.3) * 1024, "profiles/sample_rows_bf16_B64-1024_V128256.txt",                     # B = 256
                     _SAMPLING_SOURCES, "3223f9174ddd6a7a"),
@@ -225,7 +225,10 @@ def backward_throughput(sampler, iters: int = 5):
     import torch
     from benchmarks.workloads import spike_logits
 
+    from rl_engine.kernels import sampling as sampling_mod
+
     n = 64 * 512
+    rows_per_launch = min(n, sampling_mod.DEFAULT_CHUNK_TOKENS)
     logits, ids = spike_logits(n, V, seed=0, device="cuda")
     grad = torch.ones(n, device="cuda")
     logp = sampler.compute_logp(logits, ids)
@@ -244,8 +247,9 @@ def backward_throughput(sampler, iters: int = 5):
     return {"config": "bf16 logits [64,512,128256], gradient written in place; 4*V + 16 bytes per token",
             "ms": ms, "tokens_per_s": n / (ms * 1e-3),
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": gbps / HBM_PEAK_GBPS, **traffic_fields("logprob_backward_rows"),
-                         "kernel": "logprob_backward_rows<Bf16,1024,4,vec>", "bytes_per_launch": 8192 * (4 * V + 16)}}
+                         "frac": gbps / HBM_PEAK_GBPS, **traffic_fields("logprob_backward_rows", rows_per_launch / 32768),
+                         "kernel": "logprob_backward_rows<Bf16,1024,4,vec>", "rows_per_launch": rows_per_launch,
+                         "bytes_per_launch": rows_per_launch * (4 * V + 16)}}
 
 
 def lmhead_throughput(sampler, iters: int = 3):
@@ -402,7 +406,7 @@ def main() -> int:
         "pool_capacity_bytes": sampler.pool.capacity,
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS,
-                     **traffic_fields("logprob_rows", rows_per_launch / 8192),
+                     **traffic_fields("logprob_rows", rows_per_launch / 32768),
                      "kernel": "logprob_rows<Bf16,256,4,vec>", "launch_ms": launch_ms,
                      "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
     }

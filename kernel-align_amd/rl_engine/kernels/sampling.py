@@ -18,10 +18,14 @@ from rl_engine.kernels.pool import PoolExhausted, WorkspacePool
 from rl_engine.platforms.constants import constants
 from rl_engine.utils.logger import logger
 
-# Rows (tokens) per kernel launch of compute_logp.  The kernel keeps no
-# per-launch state, so this is launch granularity only: it bounds how long one
-# launch occupies the GPU and never changes a result bit.
-DEFAULT_CHUNK_TOKENS = 8192
+# Rows (tokens) per kernel launch of compute_logp and its backward.  The kernels keep no per-launch state and no
+# chunk-sized buffer, so this is launch granularity only: it bounds how long one launch occupies the GPU and never
+# changes a result bit.  Every launch ends with a tail in which the device runs empty: at V = 128,256 launches of
+# 8192 / 32768 / 131072 rows reach 6.86 / 7.01 / 7.09 TB/s.
+DEFAULT_CHUNK_TOKENS = 32768
+# Rows per chunk of the fused lm_head backward, which does hold a chunk-sized buffer ([rows, V] bf16: 2.1 GB at
+# V = 128,256).
+LMHEAD_BACKWARD_CHUNK_TOKENS = 8192
 
 _LOGPROB_FN = {torch.bfloat16: "ka_logprob_bf16", torch.float16: "ka_logprob_f16",
                torch.float32: "ka_logprob_f32"}
@@ -67,9 +71,9 @@ def _raw_stream() -> int:
     return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
-def _chunk_rows(chunk_tokens) -> int:
+def _chunk_rows(chunk_tokens, default=None) -> int:
     """Rows per launch of a chunked operator; anything below one row would make the launch loop empty."""
-    chunk = DEFAULT_CHUNK_TOKENS if chunk_tokens is None else int(chunk_tokens)
+    chunk = (DEFAULT_CHUNK_TOKENS if default is None else default) if chunk_tokens is None else int(chunk_tokens)
     if chunk < 1:
         raise ValueError(f"chunk_tokens must be >= 1 (got {chunk_tokens})")
     return chunk
@@ -480,7 +484,7 @@ class SamplerBackend(nn.Module):
             lse = lse.to(dtype=torch.float32).contiguous().view(-1)
             if w2.shape[0] % 4 != 0:  # the kernel writes four entries of a row per store: such a vocabulary keeps the GEMM path
                 lse = None
-        chunk = _chunk_rows(chunk_tokens)
+        chunk = _chunk_rows(chunk_tokens, LMHEAD_BACKWARD_CHUNK_TOKENS)
         if dweight_dtype not in (torch.float32, torch.bfloat16):
             raise TypeError("dweight_dtype must be torch.float32 or torch.bfloat16")
         dhidden = torch.empty_like(h2)
