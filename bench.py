@@ -38,7 +38,7 @@ _SAMPLING_SOURCES = ("ka_common.h", "ka_sampling_common.h", "ka_sampling_topk.h"
                      "ka_sampling_kernel.h", "ka_sampling.hip", "ka_sampling_half.hip")
 _LMHEAD_SOURCES = ("ka_common.h", "ka_lmhead.hip", "ka_lmhead_narrow.h")
 STATIC_TRAFFIC = {
-    "logprob_rows": ((2 * 4106340 + 1054.3) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",           # 32768 rows
+    "logprob_rows": ((2 * 16425200 + 4339.2) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",         # 131072 rows
                      ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
     "logprob_backward_rows": ((2 * 4108350 + 8208390) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",  # 32768 rows
                               ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
@@ -406,7 +406,7 @@ def main() -> int:
         "pool_capacity_bytes": sampler.pool.capacity,
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS,
-                     **traffic_fields("logprob_rows", rows_per_launch / 32768),
+                     **traffic_fields("logprob_rows", rows_per_launch / 131072),
                      "kernel": "logprob_rows<Bf16,256,4,vec>", "launch_ms": launch_ms,
                      "bytes_per_launch": rows_per_launch * BYTES_PER_TOKEN},
     }

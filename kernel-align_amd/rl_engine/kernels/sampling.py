@@ -21,8 +21,8 @@ from rl_engine.utils.logger import logger
 # Rows (tokens) per kernel launch of compute_logp and its backward.  The kernels keep no per-launch state and no
 # chunk-sized buffer, so this is launch granularity only: it bounds how long one launch occupies the GPU and never
 # changes a result bit.  Every launch ends with a tail in which the device runs empty: at V = 128,256 launches of
-# 8192 / 32768 / 131072 rows reach 6.86 / 7.01 / 7.09 TB/s.
-DEFAULT_CHUNK_TOKENS = 32768
+# 8192 / 32768 / 131072 rows reach 6.86 / 7.01 / 7.09 TB/s, so the default is a large group (256 x 512 tokens).
+DEFAULT_CHUNK_TOKENS = 131072
 # Rows per chunk of the fused lm_head backward, which does hold a chunk-sized buffer ([rows, V] bf16: 2.1 GB at
 # V = 128,256).
 LMHEAD_BACKWARD_CHUNK_TOKENS = 8192
