@@ -97,6 +97,29 @@ def test_generate_loop_matches_stepwise_oracle():
     assert done.any()
 
 
+def test_large_batch_sampling_replayed_from_a_hip_graph(sampler):
+    """A batch of more rows than the device has CUs runs the short top-k route with two rows resident per CU: captured and
+    replayed, ids and policy log-probabilities equal the eager call's and the oracle's ids."""
+    from oracle import exact
+
+    slog, u = cfg5_sampling(600, device="cuda", vocab=32000)
+    eager = sampler.sample(slog, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ids, pol = sampler.sample(slog, top_k=50, top_p=0.9, temperature=0.7, uniforms=u, return_policy_logprob=True)
+    for _ in range(3):
+        with torch.inference_mode():
+            ids.zero_(); pol.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ids, eager[0]) and torch.equal(pol.view(torch.int32), eager[1].view(torch.int32))
+        junk = torch.randn(1 << 18, device="cuda").sum().item()          # eager work between replays
+        assert junk == junk
+    assert torch.equal(ids.cpu(), exact.sample(slog.cpu(), 0.7, 50, 0.9, u.cpu()))
+
+
 def test_decode_step_replayed_from_a_hip_graph(sampler):
     """GraphedDecodeStep records sample + compute_logp once and replays them: every replay - with the program's own
     eager work and synchronisations between them - must give the eager operators' results bit for bit, and those
