@@ -150,8 +150,14 @@ def test_bit_identical_across_runs_and_row_counts(sampler):
     h, w, i = hidden.cuda(), weight.cuda(), ids.cuda()
     base = sampler.fused_linear_logp(h, w, i)
     assert torch.equal(base, sampler.fused_linear_logp(h, w, i))
-    for n in (1, 255, 256, 1024):
-        assert torch.equal(base[:n], sampler.fused_linear_logp(h[:n], w, i[:n]))
+    # 1 .. 64 rows: the 64-token kernel; 65 .. 128: the 128-token kernel; above: the 256-token kernel (with units as work
+    # items while token blocks x splits < 256: every call here; the test at the benchmark shape crosses into whole splits)
+    for n in (1, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 1024, 1281):
+        assert torch.equal(base[:n], sampler.fused_linear_logp(h[:n], w, i[:n])), n
+    lp, ent = sampler.fused_linear_logp(h, w, i, return_entropy=True)
+    for n in (63, 65, 128, 300):
+        lp_n, ent_n = sampler.fused_linear_logp(h[100:100 + n], w, i[100:100 + n], return_entropy=True)
+        assert torch.equal(lp_n, base[100:100 + n]) and torch.equal(ent_n, ent[100:100 + n]), n
     assert torch.equal(base[600:900], sampler.fused_linear_logp(h[600:900], w, i[600:900]))
 
 
