@@ -37,7 +37,7 @@ extern "C" {
 #define KA_DTYPE_F16 1
 #define KA_DTYPE_F32 2
 
-/* Library version string, e.g. "kernel_align_hip 0.3 (gfx950)". */
+/* Library version string, e.g. "kernel_align_hip 0.4 (gfx950)". */
 const char *ka_version(void);
 /*
  * Revision of this interface: raised whenever the signature or the meaning of an entry point changes.  A binding
@@ -46,7 +46,7 @@ const char *ka_version(void);
  * Result bits of the floating-point operators (fixed summation orders) are stable within one revision of the library,
  * not across revisions; token ids are defined exactly and never change.
  */
-#define KA_ABI_REVISION 3
+#define KA_ABI_REVISION 4
 int ka_abi_revision(void);
 /* Message of the last error on the calling thread ("" if none). */
 const char *ka_last_error(void);

@@ -23,7 +23,7 @@ int check_hip(hipError_t err, const char *what) {
 
 }  // namespace ka
 
-KA_EXPORT const char *ka_version(void) { return "kernel_align_hip 0.3 (gfx950)"; }
+KA_EXPORT const char *ka_version(void) { return "kernel_align_hip 0.4 (gfx950)"; }
 
 KA_EXPORT int ka_abi_revision(void) { return KA_ABI_REVISION; }
 

@@ -41,14 +41,18 @@ __device__ __forceinline__ void fold(RowState &st, const float (&x)[N]) {
 #pragma unroll
     for (int j = 0; j < N; ++j) e[j] = fast_exp2(fmaf(x[j], kLog2e, -ml2n));
     if (ENTROPY) {
-        float w[N];
+        // sum of x * e in four chains of FMAs (element j goes to chain j % 4); x is clamped to a finite value first, so
+        // that a masked entry (-inf, e = 0) adds 0 and not 0 * inf
+        constexpr int CHAINS = N < 4 ? N : 4;
+        float w[CHAINS];
 #pragma unroll
-        for (int j = 0; j < N; ++j) w[j] = (e[j] == 0.0f) ? 0.0f : x[j] * e[j];  // 0 * -inf stays 0
+        for (int c = 0; c < CHAINS; ++c) w[c] = 0.0f;
 #pragma unroll
-        for (int step = 1; step < N; step <<= 1)
-#pragma unroll
-            for (int j = 0; j + step < N; j += 2 * step) w[j] += w[j + step];
-        st.a = fmaf(st.a, rescale, w[0]);
+        for (int j = 0; j < N; ++j) w[j % CHAINS] = fmaf(fmaxf(x[j], -3.0e38f), e[j], w[j % CHAINS]);
+        float sum = w[0];
+        if (CHAINS == 4) sum = (w[0] + w[1]) + (w[2] + w[3]);
+        else if (CHAINS == 2) sum = w[0] + w[1];
+        st.a = fmaf(st.a, rescale, sum);
     }
     // Pairwise tree in a fixed order.
 #pragma unroll

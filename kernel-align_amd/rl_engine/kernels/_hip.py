@@ -17,7 +17,7 @@ KA_ERR_WORKSPACE = -3
 KA_ERR_HIP = -4
 
 # Revision of include/kernel_align_hip.h that the signatures below were written against (KA_ABI_REVISION).
-ABI_REVISION = 3
+ABI_REVISION = 4
 
 LIB_NAME = "libkernel_align_hip.so"
 ENV_LIB = "KERNEL_ALIGN_HIP_LIB"
