@@ -38,10 +38,10 @@ _SAMPLING_SOURCES = ("ka_common.h", "ka_sampling_common.h", "ka_sampling_topk.h"
                      "ka_sampling_kernel.h", "ka_sampling.hip", "ka_sampling_half.hip")
 _LMHEAD_SOURCES = ("ka_common.h", "ka_lmhead.hip", "ka_lmhead_narrow.h")
 STATIC_TRAFFIC = {
-    "logprob_rows": ((2 * 16425200 + 4339.2) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",         # 131072 rows
-                     ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
+    "logprob_rows": ((2 * 16425200 + 4317.5) * 1024, "profiles/logprob_rows_bf16_G256_L512_V128256.txt",         # 131072 rows
+                     ("ka_common.h", "ka_logprob.hip"), "d3ed0936386075a5"),
     "logprob_backward_rows": ((2 * 4108350 + 8208390) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",  # 32768 rows
-                              ("ka_common.h", "ka_logprob.hip"), "d51491dc6263fd14"),
+                              ("ka_common.h", "ka_logprob.hip"), "d3ed0936386075a5"),
     "sample_rows": ((2 * 32856.4 + 10.3) * 1024, "profiles/sample_rows_bf16_B64-1024_V128256.txt",                     # B = 256
                     _SAMPLING_SOURCES, "3223f9174ddd6a7a"),
     "lmhead_partials": ((2 * 3.176e7 + 121088) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt",            # N = 32768; L2 misses: varies +-50 % between calls
