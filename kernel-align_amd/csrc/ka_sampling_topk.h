@@ -273,15 +273,19 @@ __device__ __forceinline__ int fast_topk(Shared &sh, const typename T::raw_t *rp
     //    temperature folds too many values together
     auto widen_bound = [&](uint32_t &bound) {
         if (!has_t) return true;
-        const uint32_t ty = elem_key<T>(raw_of_key<T>(bound), temp, true);
-        int guard = 0;
-        while (bound >= key_step<T>() && guard < 64) {
-            const uint32_t prev = bound - key_step<T>();
-            if (elem_key<T>(raw_of_key<T>(prev), temp, true) < ty) break;
-            bound = prev;
-            ++guard;
-        }
-        return guard < 64;
+        // Lane l scales the value l steps below the bound; scaling is monotone, so the lanes whose scaled value still
+        // equals the bound's form a prefix, and its length says how far the bound moves.  (One division per lane instead of
+        // a loop of dependent ones; every wavefront does the same work.)  All 64 lanes equal: a huge temperature.
+        const int l = tid & (kWave - 1);
+        const uint32_t mine = bound - uint32_t(l) * key_step<T>();
+        const bool valid = bound >= uint32_t(l) * key_step<T>();
+        const uint32_t key = elem_key<T>(raw_of_key<T>(valid ? mine : bound), temp, true);
+        const uint32_t ty = uint32_t(__builtin_amdgcn_readfirstlane(int(key)));
+        const uint64_t same = __ballot(valid && key >= ty);
+        if (~same == 0) return false;
+        const int n = __ffsll((long long)~same) - 1;  // length of the prefix; >= 1: lane 0
+        bound -= uint32_t(n - 1) * key_step<T>();
+        return true;
     };
     // the top_k-th largest of the 1024 lane maxima, by the same MSB-first descent over count histograms as the radix path
     auto radix_bound = [&]() -> uint32_t {
