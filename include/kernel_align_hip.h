@@ -172,7 +172,7 @@ int ka_sample_topk_topp_f32(const void *logits, int64_t batch, int64_t vocab, in
  * applies; KA_SAMPLE_FLAG_BLOCK_WIDE_TOPK keeps the top-k route on its block-wide selection and tail instead of the
  * short ones it takes for top_k <= 256 (bound from pooled maxima up to top_k = 64, from a radix descent above).  Ids
  * and log-probabilities do not depend on the flags.  KA_SAMPLE_FLAG_TWO_ROWS_PER_CU / KA_SAMPLE_FLAG_ONE_ROW_PER_CU: the
- * short top-k route (scalar top_k <= 256, 16-byte aligned 16-bit rows of at most 131,072 entries) exists on 512 and on
+ * short top-k route (scalar top_k <= 256, 16-byte aligned rows of at most 131,072 16-bit or 262,144 fp32 entries) exists on 512 and on
  * 1024 threads per row; the library takes 512, with two rows resident per CU, for batches of more rows than the device has
  * CUs, and these flags force either where the row qualifies (both give the same ids and the same log-probability bits).
  */

@@ -127,12 +127,13 @@ int launch(const void *logits, int64_t batch, int64_t vocab, int64_t row_stride,
         return check_hip(hipGetLastError(), "sample launch");
       }
     }
-    if constexpr (T::kBytes == 2) {
+    {
         // Short top-k route on a batch of more rows than CUs: 512 threads per row, two rows resident per CU (one
         // row's selection runs under the other row's read).  Up to one row per CU the 1024-thread workgroup reads its
         // row faster.  The flags force either build where the row qualifies.
         const bool k_short = prm.top_k_rows == nullptr && prm.top_k > 0 && prm.top_k < vocab && prm.top_k <= SHORT_TOPK;
-        const bool fits = aligned && vocab / T::kPerVec <= 32 * 512;  // a slot maximum per vector and lane
+        // a slot maximum per vector and lane (16-bit rows), or per group of up to four vectors (fp32 rows)
+        const bool fits = aligned && vocab / T::kPerVec <= (T::kBytes == 4 ? 4 : 1) * 32 * 512;
         if (k_short && fits && path_bits == 0 && !(flags & KA_SAMPLE_FLAG_ONE_ROW_PER_CU)) {
             bool two_rows = (flags & KA_SAMPLE_FLAG_TWO_ROWS_PER_CU) != 0;
             if (!two_rows) {

@@ -26,8 +26,8 @@ struct SampleParams {
     float *out_policy;   // optional: its log-probability under the unfiltered softmax of the raw logits
 };
 
-// Launch of the 512-thread build of sample_rows<T, false> (defined in ka_sampling_half.hip); dtype is KA_DTYPE_BF16 or
-// KA_DTYPE_F16, the row is 16-byte aligned and holds at most 32 * 512 vectors.
+// Launch of the 512-thread build of sample_rows<T, false> (defined in ka_sampling_half.hip); the row is 16-byte aligned
+// and holds at most 32 * 512 vectors (16-bit dtypes) or 4 * 32 * 512 (fp32).
 hipError_t launch_sample_rows_half(int dtype, const void *logits, int64_t batch, int vocab, int64_t row_stride,
                                    const SampleParams &prm, int path_bits, hipStream_t stream);
 

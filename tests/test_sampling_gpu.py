@@ -269,7 +269,7 @@ def test_unknown_route_flag_is_refused(sampler):
                        route_flags=_hip.SAMPLE_FLAG_TWO_ROWS_PER_CU | _hip.SAMPLE_FLAG_ONE_ROW_PER_CU)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("vocab", [128256, 131072, 4096, 1000])
 def test_two_rows_per_cu_build_returns_the_same_bits(sampler, dtype, vocab):
     """The short top-k route on 512 threads per row (two rows resident per CU, what a batch of more rows than CUs gets)
