@@ -43,7 +43,7 @@ STATIC_TRAFFIC = {
     "logprob_backward_rows": ((2 * 4108350 + 8208390) * 1024, "profiles/logprob_backward_rows_bf16_G64_L512_V128256.txt",  # 32768 rows
                               ("ka_common.h", "ka_logprob.hip"), "d3ed0936386075a5"),
     "sample_rows": ((2 * 32831.5 + 10.3) * 1024, "profiles/sample_rows_bf16_B64-1024_V128256.txt",                     # B = 256
-                    _SAMPLING_SOURCES, "15a5f83dcbe76962"),
+                    _SAMPLING_SOURCES, "817959ab3c8df18c"),
     "lmhead_partials": ((2 * 3.176e7 + 121088) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt",            # N = 32768; L2 misses: varies +-50 % between calls
                         _LMHEAD_SOURCES, "793ffdf2d7810fe0"),
     "lmhead_n64": ((2 * 517332 + 256) * 1024, "profiles/lmhead_partials_bf16_H4096_V128256.txt", _LMHEAD_SOURCES, "793ffdf2d7810fe0"),
