@@ -296,6 +296,35 @@ def test_two_rows_per_cu_build_returns_the_same_bits(sampler, dtype, vocab):
             assert torch.equal(two[0].cpu(), exact.sample(logits, temp, k, p, u)), (k, p, temp)
 
 
+def test_random_shapes_and_parameters_on_both_workgroup_sizes(sampler):
+    """Forty seeded draws of (dtype, aligned vocabulary size, batch, top_k <= 256, top_p, temperature), rows with ties
+    mixed in: both builds of the short top-k route against the exact oracle, ids and filtered log-probability."""
+    rnd = torch.Generator().manual_seed(2024)
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=rnd))]
+    for case in range(40):
+        dtype = pick(DTYPES)
+        epv = 4 if dtype == torch.float32 else 8
+        vocab = epv * int(torch.randint(1, 6000, (1,), generator=rnd))
+        batch = pick([1, 3, 17, 40])
+        k = min(int(torch.randint(1, 257, (1,), generator=rnd)), vocab - 1) if vocab > 1 else None
+        p = pick([None, 0.95, 0.9, 0.5, 0.1])
+        temp = pick([1.0, 0.7, 1.3, 0.05, 20.0])
+        logits = (torch.randn(batch, vocab, generator=rnd) * pick([0.5, 3.0, 8.0]))
+        if case % 3 == 0:
+            logits = (logits * 2).round() / 2                      # heavy ties
+        logits = logits.to(dtype)
+        u = torch.rand(batch, generator=rnd)
+        if k is None:
+            continue
+        want, want_lp = exact.sample_rows(logits, temp, k, p, u)
+        for flags in (_hip.SAMPLE_FLAG_TWO_ROWS_PER_CU, _hip.SAMPLE_FLAG_ONE_ROW_PER_CU):
+            ids, lp = sampler.sample(logits.cuda(), top_k=k, top_p=p, temperature=temp, uniforms=u.cuda(),
+                                     return_logprob=True, route_flags=flags)
+            assert torch.equal(ids.cpu(), want), (case, dtype, vocab, batch, k, p, temp, flags)
+            assert (lp.cpu().double() - want_lp).abs().max().item() < 1e-5, (case, flags)
+
+
 def test_a_batch_of_more_rows_than_cus_matches_its_rows_sampled_in_small_batches(sampler):
     """The library switches to two rows per CU above one row per CU: ids and both log-probabilities of a 600-row call are
     those of the same rows in calls of 200."""
